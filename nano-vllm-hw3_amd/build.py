@@ -1,4 +1,10 @@
-"""Build libqlinear.so (HIP, gfx950) in-tree with hipcc.  No GPU is needed to build."""
+"""Build the package's HIP libraries (gfx950) in-tree with hipcc.  No GPU is needed to build.
+
+Two libraries, each from its own folder of translation units, so that a model only waits for what it runs on:
+  qlinear  csrc/*.hip         -> nanovllm/_lib/libqlinear.so   (quantized linears, Qwen3 operators, attention)
+  seqmix   csrc/seqmix/*.hip  -> nanovllm/_lib/libseqmix.so    (multi-stream residuals, short convolutions, latent
+                                                                attention, PolyNorm / clamped GLU, expert routing)
+``python build.py [--force] [qlinear|seqmix]`` builds one of them, or both without a name."""
 import os
 import shutil
 import subprocess
@@ -9,7 +15,14 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT_DIR = os.path.join(HERE, "nanovllm", "_lib")
 LIB = os.path.join(OUT_DIR, "libqlinear.so")
+SEQMIX_LIB = os.path.join(OUT_DIR, "libseqmix.so")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-fno-gpu-rdc"]
+# the packed-f32 VALU forms stay off in the newer library (plain f32 code only)
+NO_PACKED_F32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+TARGETS = {
+    "qlinear": dict(src=CSRC, lib=LIB, header="qlinear.h", flags=FLAGS, obj=""),
+    "seqmix": dict(src=os.path.join(CSRC, "seqmix"), lib=SEQMIX_LIB, header="seqmix.h", flags=FLAGS + NO_PACKED_F32, obj="seqmix_"),
+}
 
 
 def _hipcc():
@@ -26,17 +39,24 @@ def _stale(target, deps):
     return any(os.path.getmtime(d) > t for d in deps)
 
 
-def build(force=False, verbose=True):
+def build(force=False, verbose=True, target="qlinear"):
+    """Compile one library (``target`` = "qlinear" | "seqmix") or both ("all"); returns the path of the (last) library."""
+    if target == "all":
+        for name in TARGETS:
+            lib = build(force, verbose, name)
+        return lib
+    spec = TARGETS[target]
+    CSRC, LIB, FLAGS = spec["src"], spec["lib"], spec["flags"]
     os.makedirs(OUT_DIR, exist_ok=True)
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
     hipcc = _hipcc()
     headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
-    headers.append(os.path.join(HERE, "..", "include", "qlinear.h"))
-    srcs = sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))      # every translation unit of csrc/
+    headers.append(os.path.join(HERE, "..", "include", spec["header"]))
+    srcs = sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))      # every translation unit of the folder
 
     def compile_one(src):
-        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        obj = os.path.join(objdir, spec["obj"] + src.replace(".hip", ".o"))
         path = os.path.join(CSRC, src)
         if force or _stale(obj, [path] + headers):
             cmd = [hipcc] + FLAGS + ["-c", path, "-o", obj]
@@ -56,4 +76,6 @@ def build(force=False, verbose=True):
 
 
 if __name__ == "__main__":
-    print(build(force="--force" in sys.argv))
+    names = [a for a in sys.argv[1:] if not a.startswith("-")] or ["all"]
+    for name in names:
+        print(build(force="--force" in sys.argv, target=name))

@@ -1,0 +1,84 @@
+// Short causal convolution over time on every channel, added to its input, with the last taps-1 inputs of every
+// sequence carried as state between steps.
+#include "sm_common.h"
+
+namespace sm {
+
+constexpr int kMaxTaps = 16;
+
+template <typename T>
+__global__ void canon_conv_kernel(const T* __restrict__ h, const T* __restrict__ w, const T* __restrict__ state, int run,
+                                  int runs, const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
+                                  const int32_t* __restrict__ qstart, const int32_t* __restrict__ seq_slot,
+                                  T* __restrict__ out, int W, int taps) {
+    const int64_t t = blockIdx.x;
+    const int b = tok_seq[t], pos = tok_pos[t];
+    const int i = (int)t - qstart[b];                       // index of the token inside its sequence's portion
+    const T* st = state + ((size_t)seq_slot[b] * runs + run) * (size_t)(taps - 1) * W;
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < W; c += gridDim.y * blockDim.x) {
+        const float x = to_f(h[(size_t)t * W + c]);
+        float acc = to_f(w[(size_t)c * taps + taps - 1]) * x;
+        for (int j = 0; j < taps - 1; ++j) {
+            const int back = taps - 1 - j;                  // the input `back` positions ago
+            if (pos - back < 0) continue;
+            const float v = (i - back >= 0) ? to_f(h[(size_t)(t - back) * W + c]) : to_f(st[(size_t)(i + j) * W + c]);
+            acc += to_f(w[(size_t)c * taps + j]) * v;
+        }
+        out[(size_t)t * W + c] = from_f<T>(x + acc);
+    }
+}
+
+template <typename T>
+__global__ void canon_update_kernel(const T* __restrict__ h, T* __restrict__ state, int run, int runs,
+                                    const int32_t* __restrict__ qstart, const int32_t* __restrict__ seq_slot, int W, int taps) {
+    const int b = blockIdx.x;
+    const int q0 = qstart[b], n = qstart[b + 1] - q0;
+    if (n <= 0) return;
+    T* st = state + ((size_t)seq_slot[b] * runs + run) * (size_t)(taps - 1) * W;
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < W; c += gridDim.y * blockDim.x) {
+        T nv[kMaxTaps];
+        for (int k = 0; k < taps - 1; ++k) {
+            const int src = n - (taps - 1) + k;             // index inside the portion of the input that lands at k
+            nv[k] = src >= 0 ? h[(size_t)(q0 + src) * W + c] : st[(size_t)(k + n) * W + c];
+        }
+        for (int k = 0; k < taps - 1; ++k) st[(size_t)k * W + c] = nv[k];
+    }
+}
+
+}  // namespace sm
+
+using namespace sm;
+
+extern "C" int sm_canon_conv(int dtype, const void* h, const void* w, const void* state, int run, int runs,
+                             const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* qstart, const int32_t* seq_slot,
+                             void* out, int64_t T, int W, int taps, void* stream) {
+    if (T < 0 || W < 1 || taps < 1 || run < 0 || run >= runs ||
+        (T > 0 && (!h || !w || !out || !tok_seq || !tok_pos || !qstart || !seq_slot || (taps > 1 && !state)))) {
+        set_error("sm_canon_conv: bad argument");
+        return SM_EINVAL;
+    }
+    if (taps > kMaxTaps) { set_error("sm_canon_conv: at most %d taps", kMaxTaps); return SM_ESHAPE; }
+    if (T == 0) return SM_OK;
+    dim3 grid((unsigned)T, (unsigned)((W + 255) / 256));
+    SM_DISPATCH(dtype, "sm_canon_conv",
+                hipLaunchKernelGGL(canon_conv_kernel<DT>, grid, dim3(256), 0, as_stream(stream), (const DT*)h, (const DT*)w,
+                                   (const DT*)state, run, runs, tok_seq, tok_pos, qstart, seq_slot, (DT*)out, W, taps));
+    SM_CHECK_LAUNCH("sm_canon_conv");
+    return SM_OK;
+}
+
+extern "C" int sm_canon_update(int dtype, const void* h, void* state, int run, int runs, const int32_t* qstart,
+                               const int32_t* seq_slot, int B, int W, int taps, void* stream) {
+    if (B < 0 || W < 1 || taps < 1 || run < 0 || run >= runs || (B > 0 && taps > 1 && (!h || !state || !qstart || !seq_slot))) {
+        set_error("sm_canon_update: bad argument");
+        return SM_EINVAL;
+    }
+    if (taps > kMaxTaps) { set_error("sm_canon_update: at most %d taps", kMaxTaps); return SM_ESHAPE; }
+    if (B == 0 || taps == 1) return SM_OK;
+    dim3 grid((unsigned)B, (unsigned)((W + 255) / 256));
+    SM_DISPATCH(dtype, "sm_canon_update",
+                hipLaunchKernelGGL(canon_update_kernel<DT>, grid, dim3(256), 0, as_stream(stream), (const DT*)h, (DT*)state, run,
+                                   runs, qstart, seq_slot, W, taps));
+    SM_CHECK_LAUNCH("sm_canon_update");
+    return SM_OK;
+}

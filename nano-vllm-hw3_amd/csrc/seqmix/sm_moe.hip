@@ -1,0 +1,185 @@
+// Mixture of experts: the router (softmax scores, group-limited top-k, renormalised weights) and the expert products
+// in their memory-bound form, one (token, chosen expert) pair at a time.
+#include "sm_common.h"
+
+namespace sm {
+
+constexpr int kMaxExperts = 1024, kMaxTop = 32;
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, const float* __restrict__ router_w,
+                                                        int32_t* __restrict__ idx, float* __restrict__ wts, int W, int E, int top,
+                                                        int groups, int keep) {
+    extern __shared__ float z[];                 // E scores, then `groups` group scores
+    const int64_t t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const T* hr = h + (size_t)t * W;
+    for (int e = wave; e < E; e += 4) {
+        const float* wr = router_w + (size_t)e * W;
+        float d = 0.f;
+        for (int c = lane; c < W; c += 64) d += to_f(hr[c]) * wr[c];
+        d = wave_sum(d);
+        if (lane == 0) z[e] = d;
+    }
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+    // one thread finishes the token: E is small and the selections are sequential by nature
+    float mx = -INFINITY;
+    for (int e = 0; e < E; ++e) mx = fmaxf(mx, z[e]);
+    float sum = 0.f;
+    for (int e = 0; e < E; ++e) { z[e] = expf(z[e] - mx); sum += z[e]; }
+    const float inv = 1.f / sum;
+    for (int e = 0; e < E; ++e) z[e] *= inv;
+    float* gs = z + E;
+    if (groups > 1) {
+        const int per = E / groups;
+        for (int g = 0; g < groups; ++g) {
+            float m = -1.f;
+            for (int e = 0; e < per; ++e) m = fmaxf(m, z[g * per + e]);
+            gs[g] = m;
+        }
+        // mark the best `keep` groups by negating the others' score; a dropped group's experts become ineligible
+        for (int k = 0; k < keep; ++k) {
+            int best = -1;
+            float bv = -1.f;
+            for (int g = 0; g < groups; ++g)
+                if (gs[g] >= 0.f && gs[g] > bv) { bv = gs[g]; best = g; }
+            if (best >= 0) gs[best] = -2.f;                     // -2 = kept
+        }
+    }
+    int chosen[kMaxTop];
+    float cw[kMaxTop];
+    float tot = 0.f;
+    for (int k = 0; k < top; ++k) {
+        int best = -1;
+        float bv = -1.f;
+        for (int e = 0; e < E; ++e) {
+            if (groups > 1 && gs[e / (E / groups)] != -2.f) continue;
+            bool taken = false;
+            for (int j = 0; j < k; ++j) taken |= chosen[j] == e;
+            if (!taken && z[e] > bv) { bv = z[e]; best = e; }
+        }
+        chosen[k] = best < 0 ? 0 : best;
+        cw[k] = best < 0 ? 0.f : bv;
+        tot += cw[k];
+    }
+    const float rn = 1.f / (tot + 1e-20f);
+    for (int k = 0; k < top; ++k) {
+        idx[(size_t)t * top + k] = chosen[k];
+        wts[(size_t)t * top + k] = cw[k] * rn;
+    }
+}
+
+__device__ __forceinline__ float clamped_glu(float g, float u, float limit, float alpha) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.f + __expf(-alpha * g)) * (u + 1.f);
+}
+
+// workgroup = one (token, expert) pair; every wave produces outputs f = wave, wave + 4, ...
+template <typename T>
+__global__ __launch_bounds__(256) void moe_pairs_gate_up_kernel(const T* __restrict__ h, const int32_t* __restrict__ idx,
+                                                                const T* __restrict__ w_gu, float limit, float alpha,
+                                                                T* __restrict__ act, int top, int W, int F) {
+    extern __shared__ float h_lds[];
+    const int64_t p = blockIdx.x, t = p / top;
+    const int e = idx[p];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int c = threadIdx.x; c < W; c += 256) h_lds[c] = to_f(h[(size_t)t * W + c]);
+    __syncthreads();
+    const T* wg = w_gu + (size_t)e * 2 * F * W;
+    for (int f = wave; f < F; f += 4) {
+        const T* g_row = wg + (size_t)f * W;
+        const T* u_row = wg + (size_t)(F + f) * W;
+        float g = 0.f, u = 0.f;
+        for (int c = lane; c < W; c += 64) {
+            const float x = h_lds[c];
+            g += x * to_f(g_row[c]);
+            u += x * to_f(u_row[c]);
+        }
+        g = wave_sum(g);
+        u = wave_sum(u);
+        // the products leave the matrix unit in the storage type, as a GEMM's output would
+        if (lane == 0) act[(size_t)p * F + f] = from_f<T>(clamped_glu(to_f(from_f<T>(g)), to_f(from_f<T>(u)), limit, alpha));
+    }
+}
+
+// workgroup = one token; every wave produces output columns w = wave, wave + 4, ...
+template <typename T>
+__global__ __launch_bounds__(256) void moe_pairs_down_kernel(const T* __restrict__ act, const int32_t* __restrict__ idx,
+                                                             const float* __restrict__ wts, const T* __restrict__ w_down,
+                                                             const T* __restrict__ shared, T* __restrict__ y, int top, int W, int F) {
+    extern __shared__ float a_lds[];             // top * F activations of the token's pairs
+    const int64_t t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int c = threadIdx.x; c < top * F; c += 256) a_lds[c] = to_f(act[(size_t)t * top * F + c]);
+    __syncthreads();
+    for (int w = wave; w < W; w += 4) {
+        float tot = 0.f;
+        for (int k = 0; k < top; ++k) {
+            const int e = idx[(size_t)t * top + k];
+            const T* row = w_down + ((size_t)e * W + w) * F;
+            float d = 0.f;
+            for (int c = lane; c < F; c += 64) d += a_lds[k * F + c] * to_f(row[c]);
+            d = wave_sum(d);
+            tot += wts[(size_t)t * top + k] * to_f(from_f<T>(d));
+        }
+        if (lane == 0) {
+            if (shared) tot += to_f(shared[(size_t)t * W + w]);
+            y[(size_t)t * W + w] = from_f<T>(tot);
+        }
+    }
+}
+
+}  // namespace sm
+
+using namespace sm;
+
+extern "C" int sm_moe_route(int dtype, const void* h, const float* router_w, int32_t* idx, float* wts, int64_t T, int W, int E,
+                            int top, int groups, int keep, void* stream) {
+    if (T < 0 || W < 1 || E < 1 || top < 1 || (T > 0 && (!h || !router_w || !idx || !wts))) {
+        set_error("sm_moe_route: bad argument");
+        return SM_EINVAL;
+    }
+    if (groups < 1) groups = 1;
+    if (E > kMaxExperts || top > kMaxTop || top > E || E % groups || keep < 1 || keep > groups || top > keep * (E / groups)) {
+        set_error("sm_moe_route: unsupported routing shape (E=%d top=%d groups=%d keep=%d)", E, top, groups, keep);
+        return SM_ESHAPE;
+    }
+    if (T == 0) return SM_OK;
+    SM_DISPATCH(dtype, "sm_moe_route",
+                hipLaunchKernelGGL(moe_route_kernel<DT>, dim3((unsigned)T), dim3(256), (size_t)(E + groups) * 4, as_stream(stream),
+                                   (const DT*)h, router_w, idx, wts, W, E, top, groups, keep));
+    SM_CHECK_LAUNCH("sm_moe_route");
+    return SM_OK;
+}
+
+extern "C" int sm_moe_pairs_gate_up(int dtype, const void* h, const int32_t* idx, const void* w_gu, float limit, float alpha,
+                                    void* act, int64_t T, int top, int W, int F, void* stream) {
+    if (T < 0 || top < 1 || W < 1 || F < 1 || (T > 0 && (!h || !idx || !w_gu || !act))) {
+        set_error("sm_moe_pairs_gate_up: bad argument");
+        return SM_EINVAL;
+    }
+    if ((size_t)W * 4 > 60000) { set_error("sm_moe_pairs_gate_up: width too large"); return SM_ESHAPE; }
+    if (T == 0) return SM_OK;
+    SM_DISPATCH(dtype, "sm_moe_pairs_gate_up",
+                hipLaunchKernelGGL(moe_pairs_gate_up_kernel<DT>, dim3((unsigned)(T * top)), dim3(256), (size_t)W * 4,
+                                   as_stream(stream), (const DT*)h, idx, (const DT*)w_gu, limit, alpha, (DT*)act, top, W, F));
+    SM_CHECK_LAUNCH("sm_moe_pairs_gate_up");
+    return SM_OK;
+}
+
+extern "C" int sm_moe_pairs_down(int dtype, const void* act, const int32_t* idx, const float* wts, const void* w_down,
+                                 const void* shared, void* y, int64_t T, int top, int W, int F, void* stream) {
+    if (T < 0 || top < 1 || W < 1 || F < 1 || (T > 0 && (!act || !idx || !wts || !w_down || !y))) {
+        set_error("sm_moe_pairs_down: bad argument");
+        return SM_EINVAL;
+    }
+    if ((size_t)top * F * 4 > 60000) { set_error("sm_moe_pairs_down: top * F too large"); return SM_ESHAPE; }
+    if (T == 0) return SM_OK;
+    SM_DISPATCH(dtype, "sm_moe_pairs_down",
+                hipLaunchKernelGGL(moe_pairs_down_kernel<DT>, dim3((unsigned)T), dim3(256), (size_t)top * F * 4, as_stream(stream),
+                                   (const DT*)act, idx, wts, (const DT*)w_down, (const DT*)shared, (DT*)y, top, W, F));
+    SM_CHECK_LAUNCH("sm_moe_pairs_down");
+    return SM_OK;
+}

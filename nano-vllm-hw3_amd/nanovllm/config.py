@@ -11,6 +11,17 @@ def load_hf_config(model_dir: str) -> SimpleNamespace:
     """config.json -> attribute namespace (no dependency on a particular transformers version)."""
     with open(os.path.join(model_dir, "config.json")) as f:
         d = json.load(f)
+    from nanovllm.models import registry
+    arch = registry.architecture_of(d)
+    normalize = getattr(registry.model_class(arch), "normalize_config", None)
+    if normalize is not None:
+        # a model family with its own config.json layout brings it to the fields the engine reads
+        d = normalize(d)
+        d["architecture_name"] = arch
+        dt = d.get("torch_dtype", "bfloat16")
+        d["torch_dtype"] = getattr(torch, dt) if isinstance(dt, str) else dt
+        return SimpleNamespace(**d)
+    d["architecture_name"] = arch
     rope_theta = d.get("rope_theta")
     if rope_theta is None:
         rope_theta = (d.get("rope_parameters") or {}).get("rope_theta", 1000000.0)
@@ -41,7 +52,7 @@ class Config:
     enforce_eager: bool = False
     hf_config: Optional[SimpleNamespace] = None
     eos: int = -1
-    kvcache_block_size: int = 256
+    kvcache_block_size: int = 0        # 0 = the model family's own (256 for the paged K/V cache, 64 for latent caches)
     num_kvcache_blocks: int = -1
     linear_dtype: torch.dtype = torch.bfloat16
     weight_quant_fn: Optional[Callable[[torch.Tensor], torch.Tensor]] = None
@@ -54,14 +65,31 @@ class Config:
     # "cuda" = the product path (HIP kernels).  "cpu" = plumbing only: the UNQUANTIZED model with plain torch
     # operators, eager, for checking engine wiring on a host without a GPU; every quantized option is refused there.
     device: str = "cuda"
+    # compute and storage type of the model; None = what config.json says (bfloat16 if it says nothing)
+    dtype: Optional[torch.dtype] = None
+    # models that are stepped with portions of sequences (prompt pieces beside decoded tokens in one batch):
+    # the most tokens of one sequence in one step (0 = only the step's token budget limits a portion)
+    prefill_chunk: int = 0
 
     def __post_init__(self):
         assert os.path.isdir(self.model), f"{self.model} is not a directory"
-        assert self.kvcache_block_size % 256 == 0
         assert 1 <= self.tensor_parallel_size <= 8
         self.hf_config = load_hf_config(self.model)
+        if self.dtype is not None:
+            self.hf_config.torch_dtype = self.dtype
+        from nanovllm.models import registry
+        cls = registry.model_class(self.hf_config.architecture_name)
+        self.runs_portions = bool(getattr(cls, "runs_portions", False))
+        if self.kvcache_block_size == 0:
+            self.kvcache_block_size = getattr(cls, "default_block_size", 256)
+        assert self.kvcache_block_size % (64 if self.runs_portions else 256) == 0
         self.max_model_len = min(self.max_model_len, self.hf_config.max_position_embeddings)
-        assert self.max_num_batched_tokens >= self.max_model_len
+        # (a model stepped with portions cuts a long prompt over several steps)
+        assert self.runs_portions or self.max_num_batched_tokens >= self.max_model_len
+        if self.runs_portions:
+            assert self.tensor_parallel_size == 1, "this model family runs on one GPU"
+            assert self.quant_type is None and self.weight_quant_fn is None and self.load_format != "quantized", \
+                "the quantized linears are wired into the Qwen3 decoder only"
         assert self.device in ("cuda", "cpu")
         if self.device == "cpu":
             quantized = (self.quant_type is not None or self.weight_quant_fn is not None or self.quantize_lm_head or

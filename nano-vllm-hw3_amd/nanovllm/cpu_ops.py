@@ -82,3 +82,110 @@ def paged_attn_decode(q, k_cache, v_cache, block_tables, context_lens, scale):
 
 def argmax_rows(logits):
     return logits.float().argmax(-1)
+
+
+# ---- plumbing counterparts of nanovllm/seq_ops.py -------------------------------------------------------------------
+def embed_streams(ids, positions, embed, pos_table, streams):
+    x = embed[ids].float()
+    if pos_table is not None:
+        x = x + pos_table[positions.long()].float()
+    return x[:, None, :].repeat(1, streams, 1).contiguous()
+
+
+def stream_step(X, y, mix, out, w_in, norm_w, eps, dtype):
+    if y is not None:
+        X.copy_(torch.einsum("sr,tsw->trw", mix, X) + out[None, :, None] * y.float()[:, None, :])
+    if w_in is None:
+        return None
+    u = torch.einsum("s,tsw->tw", w_in, X)
+    return (u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()).to(dtype)
+
+
+def canon_conv(h, w, state, run, ctx):
+    taps = w.shape[1]
+    out = torch.empty_like(h)
+    qs = ctx.qstart.tolist()
+    for b in range(ctx.num_seqs):
+        a, e = qs[b], qs[b + 1]
+        if e <= a:
+            continue
+        slot, pos0 = int(ctx.seq_slot[b]), int(ctx.seq_pos0[b])
+        prev = state[slot, run].float().clone()                     # [taps-1, W]: inputs at pos0-(taps-1) .. pos0-1
+        for k in range(taps - 1):
+            if pos0 - (taps - 1) + k < 0:
+                prev[k] = 0
+        hist = torch.cat([prev, h[a:e].float()], 0)
+        acc = h[a:e].float().clone()
+        for j in range(taps):
+            acc += w[:, j].float() * hist[j:j + e - a]
+        out[a:e] = acc.to(h.dtype)
+        if taps > 1:
+            state[slot, run] = hist[-(taps - 1):].to(state.dtype)
+    return out
+
+
+def latent_norm_store(x, w, eps, cache, slot_mapping):
+    xf = x.float()
+    c = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(cache.dtype)
+    keep = slot_mapping >= 0
+    cache.view(-1, cache.shape[-1])[slot_mapping[keep].long()] = c[keep]
+
+
+def latent_attention(q, cache, ctx, scale):
+    o = torch.empty_like(q)
+    bs = cache.shape[1]
+    rows = cache.view(-1, cache.shape[-1])
+    qs = ctx.qstart.tolist()
+    for b in range(ctx.num_seqs):
+        a, e = qs[b], qs[b + 1]
+        if e <= a:
+            continue
+        n = int(ctx.ctx_lens[b])
+        t = torch.arange(n)
+        c = rows[ctx.block_tables[b, t // bs].long() * bs + t % bs].float()          # [n, R]
+        s = torch.einsum("thr,nr->thn", q[a:e].float(), c) * scale
+        pos = ctx.tok_pos[a:e].long()
+        s = s.masked_fill(t[None, None, :] > pos[:, None, None], float("-inf"))
+        o[a:e] = torch.einsum("thn,nr->thr", torch.softmax(s, -1), c).to(q.dtype)
+    return o
+
+
+def poly_norm(z, coef, eps):
+    zf = z.float()
+
+    def unit(v):
+        return v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+    a, b, c, e = coef.tolist()
+    return (a * unit(zf) + b * unit(zf * zf) + c * unit(zf * zf * zf) + e).to(z.dtype)
+
+
+def clamped_glu(gu, limit, alpha):
+    g, u = gu.float().chunk(2, -1)
+    g = g.clamp(max=limit)
+    u = u.clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1)).to(gu.dtype)
+
+
+def moe_route(h, router_w, top, groups, keep):
+    T, E = h.shape[0], router_w.shape[0]
+    s = torch.softmax(h.float() @ router_w.t(), -1)
+    masked = s
+    if groups > 1:
+        per = E // groups
+        best = s.view(T, groups, per).amax(-1).topk(keep, -1).indices
+        ok = torch.zeros(T, groups, dtype=torch.bool).scatter_(1, best, True)
+        masked = s.masked_fill(~ok.repeat_interleave(per, 1), -1.0)
+    idx = masked.topk(top, -1).indices
+    w = s.gather(1, idx)
+    return idx.int(), w / (w.sum(-1, keepdim=True) + 1e-20)
+
+
+def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha, shared):
+    y = torch.zeros(h.shape, dtype=torch.float32)
+    for e in idx.unique().tolist():
+        tok, k = (idx == e).nonzero(as_tuple=True)
+        act = clamped_glu(F.linear(h[tok], w_gu[e]), limit, alpha)
+        y.index_add_(0, tok, wts[tok, k][:, None] * F.linear(act, w_down[e]).float())
+    if shared is not None:
+        y = y + shared.float()
+    return y.to(h.dtype)

@@ -33,3 +33,40 @@ class BlockManager:
     def may_append(self, seq):
         if len(seq) % self.block_size == 1 and len(seq.block_table) < self._needed(seq):
             seq.block_table.append(self.free.popleft())
+
+    # ---- growth by portions (models whose prompts are cached piece by piece)
+    def blocks_short(self, seq, num_tokens: int) -> int:
+        """How many more blocks the sequence needs to hold ``num_tokens`` tokens."""
+        return max(0, (num_tokens + self.block_size - 1) // self.block_size - len(seq.block_table))
+
+    def reserve(self, seq, num_tokens: int) -> bool:
+        """Grow the sequence's block table to hold ``num_tokens`` tokens; False (and nothing taken) if the pool cannot."""
+        need = self.blocks_short(seq, num_tokens)
+        if need > len(self.free):
+            return False
+        for _ in range(need):
+            seq.block_table.append(self.free.popleft())
+        return True
+
+
+class SlotPool:
+    """Fixed-size per-sequence state (the carried inputs of short convolutions, recurrent state) lives in numbered
+    slots of one tensor; a sequence holds a slot from its first step until it ends or is preempted.  A slot is NOT
+    cleared when it changes hands: the kernels never read state that lies before a sequence's first token."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots
+        self.free = deque(range(num_slots))
+
+    def acquire(self, seq) -> bool:
+        if seq.state_slot >= 0:
+            return True
+        if not self.free:
+            return False
+        seq.state_slot = self.free.popleft()
+        return True
+
+    def release(self, seq):
+        if seq.state_slot >= 0:
+            self.free.append(seq.state_slot)
+            seq.state_slot = -1

@@ -58,6 +58,23 @@ class LLMEngine:
         num_tokens = sum(len(s) for s in seqs) if is_prefill else -len(seqs)
         return outputs, num_tokens
 
+    # ------------------------------------------------------------------ models stepped with portions
+    def forward_portions(self, batch, rows=None):
+        """The engine's step for a model that is stepped with portions: ``batch`` = [(sequence, token count)], each
+        sequence already holding its state slot and cache blocks (Scheduler.reserve_portion).  Runs the tokens,
+        returns float32 logits (of ``rows`` of the packed step, default every portion's last token) and marks nothing:
+        the caller commits (sampling) or advances the sequences itself (replaying given tokens)."""
+        return self.model_runner.run_portions(batch, rows)
+
+    def step_portions(self):
+        """schedule -> run -> greedy sample -> commit; returns the finished sequences' (id, completion tokens)."""
+        sch = self.scheduler
+        batch = sch.schedule_portions()
+        logits = self.forward_portions(batch)
+        tokens = logits.argmax(dim=-1).tolist()
+        done = sch.commit_portions(batch, {seq.seq_id: tok for (seq, _), tok in zip(batch, tokens)})
+        return [(s.seq_id, s.completion_token_ids) for s in done]
+
     def _can_pipeline(self):
         """The next step may be launched before the tokens of the one in flight are known if it can only be a
         decode step over a subset of the same sequences: nothing is waiting for prefill, every running sequence
@@ -76,6 +93,13 @@ class LLMEngine:
             self.add_request(p, sp)
         outputs = {}
         sch, runner = self.scheduler, self.model_runner
+        if sch.portions:
+            while not self.is_finished():
+                for seq_id, toks in self.step_portions():
+                    outputs[seq_id] = toks
+            outs = [outputs[k] for k in sorted(outputs)]
+            decode = (lambda t: self.tokenizer.decode(t)) if self.tokenizer is not None else (lambda t: "")
+            return [{"text": decode(t), "token_ids": t} for t in outs]
         pending = None                      # (seqs, token indices, handle, covers) of the step in flight
 
         def drain(p):

@@ -6,7 +6,8 @@ import torch.distributed as dist
 
 from nanovllm.config import Config
 from nanovllm.engine.sequence import Sequence
-from nanovllm.models.qwen3 import AttnContext, Qwen3ForCausalLM, set_context
+from nanovllm.models import registry
+from nanovllm.models.qwen3 import AttnContext, set_context
 from nanovllm.utils.loader import init_dummy_weights, load_model
 from nanovllm.utils.quantization import apply_quant_from_config, reserve_workspace
 
@@ -25,7 +26,12 @@ class ModelRunner:
         torch.set_default_dtype(hf.torch_dtype)
         torch.set_default_device(self.device)
         try:
-            self.model = Qwen3ForCausalLM(hf)
+            model_cls = registry.model_class(hf.architecture_name)
+            self.portions = bool(getattr(model_cls, "runs_portions", False))
+            if self.portions:
+                self._init_portion_model(model_cls)
+                return
+            self.model = model_cls(hf)
             if config.load_format == "quantized":
                 # a pre-quantized checkpoint: no bf16 read, no re-quantization
                 from nanovllm.utils.checkpoint import load_quantized
@@ -67,6 +73,101 @@ class ModelRunner:
         finally:
             torch.set_default_device("cpu")
             torch.set_default_dtype(default_dtype)
+
+    # ------------------------------------------------------------------ models stepped with portions
+    def _init_portion_model(self, model_cls):
+        """A model family that is stepped with portions of sequences and owns its cache and per-sequence state: the
+        runner loads it, sizes the block pool and the state slots, and hands every step a StepContext."""
+        cfg, hf = self.config, self.config.hf_config
+        if self.on_gpu:
+            from nanovllm import _seqmix
+            _seqmix.build_if_missing()           # a fresh checkout compiles this library (and only it) here
+            _seqmix.load()
+            # float32 means float32: no reduced-precision matrix mode
+            torch.backends.cuda.matmul.allow_tf32 = False
+        self.model = model_cls(hf)
+        if cfg.load_format == "dummy":
+            init_dummy_weights(self.model, hf, seed=0)
+        else:
+            load_model(self.model, cfg.model)
+        bs, slots = self.block_size, cfg.max_num_seqs
+        block_bytes = self.model.cache_bytes_per_block(bs)
+        if self.on_gpu:
+            free, total = torch.cuda.mem_get_info()
+            budget = int(free - (1.0 - cfg.gpu_memory_utilization) * total) - (10 << 30) - slots * self.model.state_bytes_per_slot()
+        else:
+            budget = 1 << 30
+        max_needed = cfg.max_num_seqs * ((cfg.max_model_len + bs - 1) // bs)
+        if cfg.num_kvcache_blocks > 0:            # an explicit pool size (tests, replaying a trace): taken as given
+            max_needed = cfg.num_kvcache_blocks
+        cfg.num_kvcache_blocks = max(1, min(budget // max(block_bytes, 1), max_needed))
+        self.model.allocate_cache(cfg.num_kvcache_blocks, bs, slots, self.device)
+        self._stage_max_bs = 0
+        self._stage_rows = []
+        self._tok_host = [torch.zeros(0, dtype=torch.int64)]
+
+    def prepare_portions(self, batch):
+        """[(sequence, token count)] -> (input ids, positions, StepContext).  Every index the kernels need travels in
+        ONE int32 buffer: a single host-to-device copy per step."""
+        import numpy as np
+        from nanovllm.seq_ops import StepContext
+        bs = self.block_size
+        B = len(batch)
+        T = sum(n for _, n in batch)
+        mb = max(1, max((s.num_computed + n + bs - 1) // bs for s, n in batch))
+        sizes = [2 * T, T, T, T, B + 1, B, B, B, B * mb]
+        offs = np.concatenate([[0], np.cumsum(sizes)])
+        buf = np.zeros(int(offs[-1]) + 1, dtype=np.int32)
+        ids = buf[offs[0]:offs[1]].view(np.int64)
+        tok_seq, tok_pos, slot_map = (buf[offs[i]:offs[i + 1]] for i in (1, 2, 3))
+        qstart, pos0, ctx, sslot = (buf[offs[i]:offs[i + 1]] for i in (4, 5, 6, 7))
+        tables = buf[offs[8]:offs[9]].reshape(B, mb)
+        row = 0
+        for b, (seq, n) in enumerate(batch):
+            a = seq.num_computed
+            assert n > 0 and a + n <= seq.num_tokens and seq.state_slot >= 0 and len(seq.block_table) * bs >= a + n
+            p = np.arange(a, a + n, dtype=np.int32)
+            ids[row:row + n] = seq.token_ids[a:a + n]
+            tok_seq[row:row + n] = b
+            tok_pos[row:row + n] = p
+            bt = np.asarray(seq.block_table, dtype=np.int32)
+            slot_map[row:row + n] = bt[p // bs] * bs + p % bs
+            qstart[b], pos0[b], ctx[b], sslot[b] = row, a, a + n, seq.state_slot
+            tables[b, :len(bt[:mb])] = bt[:mb]
+            row += n
+        qstart[B] = row
+        host = torch.from_numpy(buf)
+        if self.on_gpu:
+            host = host.pin_memory()
+            dev = host.to(self.device, non_blocking=True)
+        else:
+            dev = host
+        v = [dev[int(offs[i]):int(offs[i + 1])] for i in range(9)]
+        step = StepContext(tok_seq=v[1], tok_pos=v[2], slot_mapping=v[3], qstart=v[4], seq_pos0=v[5], ctx_lens=v[6],
+                           seq_slot=v[7], block_tables=v[8].view(B, mb), num_seqs=B, num_tokens=T,
+                           max_q=max(n for _, n in batch), block_size=bs, qstart_host=qstart.tolist())
+        return v[0].view(torch.int64), v[2], step
+
+    @torch.inference_mode()
+    def run_portions(self, batch, rows=None, trace=None):
+        """One step over [(sequence, token count)]: every portion's tokens run from the cache and state that earlier
+        steps left.  Returns float32 logits of ``rows`` (indices into the step's packed tokens; default: the last token
+        of every portion, in batch order)."""
+        from nanovllm import seq_ops
+        ids, pos, step = self.prepare_portions(batch)
+        seq_ops.set_step(step)
+        try:
+            h = self.model(ids, pos, trace=trace)
+        finally:
+            seq_ops.set_step(None)
+        if rows is None:
+            rows = [q - 1 for q in step.qstart_host[1:]]
+        if len(rows) == 0:
+            return torch.empty((0, self.config.hf_config.vocab_size), dtype=torch.float32, device=self.device)
+        sel = torch.tensor(rows, dtype=torch.int64)
+        if self.on_gpu:
+            sel = sel.pin_memory().to(self.device, non_blocking=True)
+        return self.model.compute_logits(h.index_select(0, sel))
 
     # ------------------------------------------------------------------ setup
     def _linear_shapes(self):

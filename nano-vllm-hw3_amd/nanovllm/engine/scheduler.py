@@ -1,6 +1,6 @@
 from collections import deque
 
-from nanovllm.engine.block_manager import BlockManager
+from nanovllm.engine.block_manager import BlockManager, SlotPool
 from nanovllm.engine.sequence import ACTIVE, DONE, QUEUED, Sequence
 
 
@@ -16,6 +16,11 @@ class Scheduler:
         self.block_manager = BlockManager(config.num_kvcache_blocks, config.kvcache_block_size)
         self.waiting = deque()
         self.running = deque()
+        # models stepped with portions: a step mixes prompt pieces and decoded tokens, and every running sequence
+        # holds a state slot besides its cache blocks
+        self.portions = bool(getattr(config, "runs_portions", False))
+        self.prefill_chunk = getattr(config, "prefill_chunk", 0) or (1 << 30)
+        self.slots = SlotPool(config.max_num_seqs if self.portions else 0)
 
     def is_finished(self):
         return not self.waiting and not self.running
@@ -119,3 +124,82 @@ class Scheduler:
 
     def postprocess(self, seqs, token_ids):
         return self.commit(seqs, self.advance(seqs), token_ids)
+
+    # ------------------------------------------------------------------ steps made of portions
+    def reserve_portion(self, seq, count: int) -> bool:
+        """Everything the next ``count`` tokens of ``seq`` need before they can run: a state slot and cache blocks up to
+        token num_computed + count.  False if the pools cannot give it (nothing is taken then, except that a slot
+        acquired for a new sequence is returned)."""
+        assert 0 < count <= seq.num_tokens - seq.num_computed
+        had_slot = seq.state_slot >= 0
+        if not self.slots.acquire(seq):
+            return False
+        if not self.block_manager.reserve(seq, seq.num_computed + count):
+            if not had_slot:
+                self.slots.release(seq)
+            return False
+        return True
+
+    def release(self, seq):
+        """Give back what a sequence holds in the cache and the state pool."""
+        self.block_manager.deallocate(seq)
+        self.slots.release(seq)
+
+    def schedule_portions(self):
+        """One step's batch as [(sequence, token count)]: every running sequence gets its next tokens first (one token
+        when it decodes, the next piece of its prompt otherwise), then waiting sequences are admitted, while the step's
+        token budget, the sequence count, the state slots and the free cache blocks allow.  When the cache cannot hold
+        the next tokens of a running sequence, the most recently admitted sequences go back to the queue."""
+        budget, batch = self.max_num_batched_tokens, []
+        for seq in list(self.running):
+            if budget == 0 or len(batch) >= self.max_num_seqs:
+                break
+            if seq.state != ACTIVE:              # preempted below while an earlier sequence was served
+                continue
+            n = min(seq.num_tokens - seq.num_computed, budget, self.prefill_chunk)
+            while not self.reserve_portion(seq, n):
+                later = [s for s in self.running if s is not seq and all(s is not b for b, _ in batch)]
+                victim = later[-1] if later else seq
+                self.preempt_portions(victim)
+                if victim is seq:
+                    break
+            if seq.state != ACTIVE:
+                continue
+            batch.append((seq, n))
+            budget -= n
+        while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs:
+            seq = self.waiting[0]
+            n = min(seq.num_tokens - seq.num_computed, budget, self.prefill_chunk)
+            if not self.reserve_portion(seq, n):
+                break
+            self.waiting.popleft()
+            seq.state = ACTIVE
+            self.running.append(seq)
+            batch.append((seq, n))
+            budget -= n
+        assert batch, "nothing to run: a single sequence does not fit the cache"
+        return batch
+
+    def preempt_portions(self, seq):
+        self.running.remove(seq)
+        self.release(seq)
+        seq.num_computed = 0
+        seq.state = QUEUED
+        self.waiting.appendleft(seq)
+
+    def commit_portions(self, batch, token_of):
+        """After a step: the portions' tokens are cached; a sequence whose known tokens are all cached receives the token
+        sampled from its last position (``token_of[seq_id]``).  Returns the sequences that finished."""
+        done = []
+        for seq, n in batch:
+            seq.num_computed += n
+            if seq.num_computed < seq.num_tokens:
+                continue
+            tok = token_of[seq.seq_id]
+            seq.append_token(tok)
+            if (not seq.ignore_eos and tok == self.eos) or seq.num_completion_tokens >= seq.max_tokens:
+                seq.state = DONE
+                self.release(seq)
+                self.running.remove(seq)
+                done.append(seq)
+        return done

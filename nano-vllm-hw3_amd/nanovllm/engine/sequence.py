@@ -13,7 +13,7 @@ QUEUED, ACTIVE, DONE = "queued", "active", "done"
 
 class Sequence:
     __slots__ = ("seq_id", "state", "token_ids", "num_tokens", "num_prompt_tokens", "last_token", "block_table",
-                 "max_tokens", "ignore_eos")
+                 "max_tokens", "ignore_eos", "num_computed", "state_slot")
 
     def __init__(self, token_ids, sampling_params: SamplingParams = None):
         sp = sampling_params if sampling_params is not None else SamplingParams()
@@ -25,6 +25,8 @@ class Sequence:
         self.num_prompt_tokens = self.num_tokens = len(ids)
         self.last_token = ids[-1]
         self.block_table = []                   # KV blocks, in order of the tokens they hold
+        self.num_computed = 0                   # tokens whose cache rows and state exist (models stepped with portions)
+        self.state_slot = -1                    # slot of per-sequence recurrent state (-1: none held)
         self.max_tokens = sp.max_tokens         # (the sampler is greedy: the temperature is not used)
         self.ignore_eos = sp.ignore_eos
 
@@ -35,6 +37,14 @@ class Sequence:
         self.token_ids.append(token_id)
         self.last_token = token_id
         self.num_tokens += 1
+
+    def extend(self, token_ids):
+        """More known tokens (a prompt that arrives in pieces)."""
+        ids = list(token_ids)
+        if ids:
+            self.token_ids.extend(ids)
+            self.num_tokens += len(ids)
+            self.last_token = ids[-1]
 
     @property
     def is_finished(self):

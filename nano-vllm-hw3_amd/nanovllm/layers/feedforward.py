@@ -1,0 +1,54 @@
+"""Feed-forward layers beyond the SiLU-gated MLP: a dense layer with the PolyNorm activation, the clamped GLU expert,
+and a routed mixture of such experts with group-limited top-k routing and an optional shared expert."""
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from nanovllm import seq_ops
+
+
+class PolyNormMLP(nn.Module):
+    """down(PolyNorm(up(h))): PolyNorm(z) = a N(z) + b N(z^2) + c N(z^3) + e with N = division by the row's RMS."""
+
+    def __init__(self, width: int, ff: int, eps: float):
+        super().__init__()
+        self.eps = eps
+        self.up = nn.Parameter(torch.empty(ff, width), requires_grad=False)
+        self.down = nn.Parameter(torch.empty(width, ff), requires_grad=False)
+        self.coef = nn.Parameter(torch.zeros(4, dtype=torch.float32), requires_grad=False)     # a, b, c, e
+
+    def forward(self, h):
+        return F.linear(seq_ops.poly_norm(F.linear(h, self.up), self.coef, self.eps), self.down)
+
+
+class ClampedGLU(nn.Module):
+    """down(g * sigmoid(alpha g) * (u + 1)) with g = min(gate(h), limit), u = clamp(up(h), +-limit); no biases."""
+
+    def __init__(self, width: int, ff: int, limit: float, alpha: float = 1.702):
+        super().__init__()
+        self.ff, self.limit, self.alpha = ff, float(limit), alpha
+        self.gate_up = nn.Parameter(torch.empty(2 * ff, width), requires_grad=False)          # gate rows, then up rows
+        self.down = nn.Parameter(torch.empty(width, ff), requires_grad=False)
+
+    def forward(self, h):
+        return F.linear(seq_ops.clamped_glu(F.linear(h, self.gate_up), self.limit, self.alpha), self.down)
+
+
+class RoutedExperts(nn.Module):
+    """Softmax router in float32; experts in ``groups`` equal groups of neighbours, only the ``keep`` groups with the
+    largest member score are eligible; the ``top`` best eligible experts run, weighted by their renormalised scores.
+    A shared expert (its own size and limit) runs for every token and is added."""
+
+    def __init__(self, width: int, experts: int, top: int, ff: int, limit: float, groups: int = 1, keep: int = 1,
+                 shared: ClampedGLU = None, alpha: float = 1.702):
+        super().__init__()
+        self.experts, self.top, self.groups, self.keep, self.limit, self.alpha = experts, top, groups, keep, float(limit), alpha
+        self.router = nn.Parameter(torch.empty(experts, width, dtype=torch.float32), requires_grad=False)
+        self.w_gu = nn.Parameter(torch.empty(experts, 2 * ff, width), requires_grad=False)
+        self.w_down = nn.Parameter(torch.empty(experts, width, ff), requires_grad=False)
+        self.shared = shared
+
+    def forward(self, h):
+        idx, wts = seq_ops.moe_route(h, self.router, self.top, self.groups, self.keep)
+        shared = self.shared(h) if self.shared is not None else None
+        return seq_ops.moe_experts(h, idx, wts, self.w_gu, self.w_down, self.limit, self.alpha, shared)

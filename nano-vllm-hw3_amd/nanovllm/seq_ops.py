@@ -1,0 +1,192 @@
+"""Operators of libseqmix behind torch tensors: the mechanisms between the matrix products of a decoder whose layers
+use multi-stream residuals, short convolutions, latent attention, PolyNorm / clamped-GLU feed-forwards and routed
+experts.  One kernel launch each on the current stream.  CPU tensors go to plain-torch counterparts
+(nanovllm/cpu_ops.py): engine plumbing on a host without a GPU, never a fallback for a GPU tensor."""
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from nanovllm import _seqmix as SM
+from nanovllm import cpu_ops
+
+
+@dataclass
+class StepContext:
+    """What one engine step's kernels need to know about its batch: B sequences contribute portions of consecutive
+    tokens (a single token when decoding), T tokens in all, packed sequence after sequence."""
+    tok_seq: torch.Tensor          # int32 [T]  index of the token's sequence in this step
+    tok_pos: torch.Tensor          # int32 [T]  position of the token in its sequence
+    qstart: torch.Tensor           # int32 [B+1] first row of every sequence's portion
+    seq_pos0: torch.Tensor         # int32 [B]  position of the portion's first token (= tokens already cached)
+    ctx_lens: torch.Tensor         # int32 [B]  tokens cached after this step
+    seq_slot: torch.Tensor         # int32 [B]  state slot of the sequence
+    slot_mapping: torch.Tensor     # int32 [T]  cache row (block * block_size + offset) every token is stored at
+    block_tables: torch.Tensor     # int32 [B, max_blocks]
+    num_seqs: int = 0
+    num_tokens: int = 0
+    max_q: int = 0                 # longest portion
+    block_size: int = 64
+    qstart_host: Optional[list] = None
+
+
+_STEP: Optional[StepContext] = None
+
+
+def set_step(ctx):
+    global _STEP
+    _STEP = ctx
+
+
+def get_step() -> StepContext:
+    return _STEP
+
+
+def _dev(t):
+    return SM.stream_ptr(t.device)
+
+
+def embed_streams(ids, positions, embed, pos_table, streams):
+    """X f32 [T, S, W]: every stream starts as embed[id] + pos_table[position]."""
+    T, W = ids.numel(), embed.shape[1]
+    if not embed.is_cuda:
+        return cpu_ops.embed_streams(ids, positions, embed, pos_table, streams)
+    X = torch.empty((T, streams, W), dtype=torch.float32, device=embed.device)
+    SM.check(SM.load().sm_embed_streams(SM.dtype_code(embed.dtype), ids.data_ptr(), positions.data_ptr(), embed.data_ptr(),
+                                        SM.ptr(pos_table), X.data_ptr(), T, streams, W, _dev(embed)))
+    return X
+
+
+def stream_step(X, y, mix, out, w_in, norm_w, eps, dtype):
+    """Write phase (y given): X <- mix^T X + out * y in place.  Read phase (w_in given): returns
+    rms_norm(sum_s w_in[s] X[:, s]) * norm_w in ``dtype``."""
+    T, S, W = X.shape
+    if not X.is_cuda:
+        return cpu_ops.stream_step(X, y, mix, out, w_in, norm_w, eps, dtype)
+    h = torch.empty((T, W), dtype=dtype, device=X.device) if w_in is not None else None
+    if y is not None:
+        SM.require_cuda(y, dtype, "y")
+    SM.check(SM.load().sm_stream_step(SM.dtype_code(dtype), X.data_ptr(), SM.ptr(y), SM.ptr(mix), SM.ptr(out), SM.ptr(w_in),
+                                      SM.ptr(norm_w), eps, SM.ptr(h), T, S, W, _dev(X)))
+    return h
+
+
+def canon_conv(h, w, state, run, ctx: StepContext):
+    """h + causal_conv(h) per channel with the sequence's carried inputs; then the state takes this step's last inputs.
+    h [T, W], w [W, taps], state [slots, runs, taps-1, W]."""
+    T, W = h.shape
+    taps = w.shape[1]
+    if not h.is_cuda:
+        return cpu_ops.canon_conv(h, w, state, run, ctx)
+    SM.require_cuda(h, w.dtype, "h")
+    out = torch.empty_like(h)
+    lib, code, runs = SM.load(), SM.dtype_code(h.dtype), state.shape[1]
+    SM.check(lib.sm_canon_conv(code, h.data_ptr(), w.data_ptr(), state.data_ptr(), run, runs, ctx.tok_seq.data_ptr(),
+                               ctx.tok_pos.data_ptr(), ctx.qstart.data_ptr(), ctx.seq_slot.data_ptr(), out.data_ptr(), T, W,
+                               taps, _dev(h)))
+    SM.check(lib.sm_canon_update(code, h.data_ptr(), state.data_ptr(), run, runs, ctx.qstart.data_ptr(),
+                                 ctx.seq_slot.data_ptr(), ctx.num_seqs, W, taps, _dev(h)))
+    return out
+
+
+def latent_norm_store(x, w, eps, cache, slot_mapping):
+    """x [T, R] (rows may be strided: a column slice of a wider product) -> rms_norm(x) * w stored at the rows of
+    ``cache`` [blocks, block_size, R] named by slot_mapping."""
+    T, R = x.shape
+    if not x.is_cuda:
+        return cpu_ops.latent_norm_store(x, w, eps, cache, slot_mapping)
+    assert x.stride(1) == 1 and x.dtype == cache.dtype == w.dtype
+    SM.check(SM.load().sm_latent_norm_store(SM.dtype_code(x.dtype), x.data_ptr(), x.stride(0), w.data_ptr(), eps,
+                                            cache.data_ptr(), slot_mapping.data_ptr(), T, R, _dev(x)))
+
+
+USE_TILES = False      # bf16 latent attention on the matrix cores where the shape allows (tests compare both forms)
+
+
+def latent_attention(q, cache, ctx: StepContext, scale, force_rows=False):
+    """Absorbed queries q [T, H, R] over the paged latent cache [blocks, block_size, R] (keys = values = cache rows),
+    causal inside each sequence -> [T, H, R]."""
+    T, H, R = q.shape
+    if not q.is_cuda:
+        return cpu_ops.latent_attention(q, cache, ctx, scale)
+    SM.require_cuda(q, cache.dtype, "q")
+    o = torch.empty_like(q)
+    lib = SM.load()
+    bs, mb = cache.shape[1], ctx.block_tables.shape[1]
+    tiles_ok = (USE_TILES and not force_rows and q.dtype == torch.bfloat16 and R % 8 == 0 and R <= 256 and bs % 64 == 0)
+    if tiles_ok and ctx.max_q == 1:
+        splits = decode_splits(ctx.num_seqs, mb * bs)
+        ws, n = SM.decode_workspace.get(q.device, lib.sm_latent_decode_workspace_bytes(T, H, R, splits))
+        SM.check(lib.sm_latent_attn_decode(q.data_ptr(), cache.data_ptr(), ctx.block_tables.data_ptr(), ctx.ctx_lens.data_ptr(),
+                                           o.data_ptr(), scale, T, H, R, bs, mb, splits, ws, n, _dev(q)))
+    elif tiles_ok:
+        SM.check(lib.sm_latent_attn_tiles(q.data_ptr(), cache.data_ptr(), ctx.block_tables.data_ptr(), ctx.qstart.data_ptr(),
+                                          ctx.seq_pos0.data_ptr(), o.data_ptr(), scale, ctx.num_seqs, ctx.max_q, H, R, bs, mb,
+                                          _dev(q)))
+    else:
+        SM.check(lib.sm_latent_attn_rows(SM.dtype_code(q.dtype), q.data_ptr(), cache.data_ptr(), ctx.block_tables.data_ptr(),
+                                         ctx.tok_seq.data_ptr(), ctx.tok_pos.data_ptr(), o.data_ptr(), scale, T, H, R, bs, mb,
+                                         _dev(q)))
+    return o
+
+
+def decode_splits(num_seqs, max_keys):
+    """Key splits of decode attention: enough workgroups to fill 256 CUs, at least 256 keys per split.  Depends only on
+    the batch size and the cache geometry, never on the sequences' lengths, so a result does not move with them."""
+    want = max(1, 512 // max(1, num_seqs))
+    return int(max(1, min(want, max_keys // 256, 64)))
+
+
+def poly_norm(z, coef, eps):
+    """a N(z) + b N(z^2) + c N(z^3) + e per row; coef = f32 [4] = a, b, c, e."""
+    if not z.is_cuda:
+        return cpu_ops.poly_norm(z, coef, eps)
+    SM.require_cuda(z, None, "z")
+    out = torch.empty_like(z)
+    SM.check(SM.load().sm_poly_norm(SM.dtype_code(z.dtype), z.data_ptr(), coef.data_ptr(), eps, out.data_ptr(),
+                                    z.shape[0], z.shape[1], _dev(z)))
+    return out
+
+
+def clamped_glu(gu, limit, alpha=1.702):
+    """gu [T, 2F] = gate | up -> min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, +-limit) + 1)."""
+    if not gu.is_cuda:
+        return cpu_ops.clamped_glu(gu, limit, alpha)
+    SM.require_cuda(gu, None, "gu")
+    T, F2 = gu.shape
+    out = torch.empty((T, F2 // 2), dtype=gu.dtype, device=gu.device)
+    SM.check(SM.load().sm_clamped_glu(SM.dtype_code(gu.dtype), gu.data_ptr(), limit, alpha, out.data_ptr(), T, F2 // 2, _dev(gu)))
+    return out
+
+
+def moe_route(h, router_w, top, groups=1, keep=1):
+    """Softmax router with group-limited top-k: (idx int32 [T, top], weights f32 [T, top]); router_w f32 [E, W]."""
+    if not h.is_cuda:
+        return cpu_ops.moe_route(h, router_w, top, groups, keep)
+    SM.require_cuda(h, None, "h")
+    SM.require_cuda(router_w, torch.float32, "router_w")
+    T, W = h.shape
+    E = router_w.shape[0]
+    idx = torch.empty((T, top), dtype=torch.int32, device=h.device)
+    wts = torch.empty((T, top), dtype=torch.float32, device=h.device)
+    SM.check(SM.load().sm_moe_route(SM.dtype_code(h.dtype), h.data_ptr(), router_w.data_ptr(), idx.data_ptr(), wts.data_ptr(),
+                                    T, W, E, top, groups, keep, _dev(h)))
+    return idx, wts
+
+
+def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702, shared=None):
+    """y[t] = sum_k wts[t, k] * expert_{idx[t, k]}(h[t]) (+ shared[t]); w_gu [E, 2F, W] (gate rows then up rows),
+    w_down [E, W, F]; an expert is a clamped GLU between its two products."""
+    if not h.is_cuda:
+        return cpu_ops.moe_experts(h, idx, wts, w_gu, w_down, limit, alpha, shared)
+    SM.require_cuda(h, w_gu.dtype, "h")
+    T, W = h.shape
+    top, F = idx.shape[1], w_down.shape[2]
+    lib, code = SM.load(), SM.dtype_code(h.dtype)
+    act = torch.empty((T * top, F), dtype=h.dtype, device=h.device)
+    y = torch.empty_like(h)
+    SM.check(lib.sm_moe_pairs_gate_up(code, h.data_ptr(), idx.data_ptr(), w_gu.data_ptr(), limit, alpha, act.data_ptr(), T, top,
+                                      W, F, _dev(h)))
+    SM.check(lib.sm_moe_pairs_down(code, act.data_ptr(), idx.data_ptr(), wts.data_ptr(), w_down.data_ptr(), SM.ptr(shared),
+                                   y.data_ptr(), T, top, W, F, _dev(h)))
+    return y

@@ -28,10 +28,15 @@ def load_model(model, path: str):
     """Read every *.safetensors under ``path``; every rank reads the full tensors and keeps its shard."""
     from safetensors import safe_open
     params = dict(model.named_parameters())
+    # a model family with its own checkpoint names places the tensors itself (merged and stacked parameters included)
+    place = getattr(model, "load_checkpoint_tensor", None)
     for file in sorted(glob(os.path.join(path, "*.safetensors"))):
         with safe_open(file, "pt", "cpu") as f:
             for name in f.keys():
-                _assign(model, params, name, f.get_tensor(name))
+                if place is not None:
+                    place(params, name, f.get_tensor(name))
+                else:
+                    _assign(model, params, name, f.get_tensor(name))
 
 
 @torch.no_grad()
@@ -40,6 +45,12 @@ def init_dummy_weights(model, cfg, seed: int = 0, std: float = 0.02):
     checkpoint are drawn in a fixed order from one seeded generator and passed through the same
     weight loaders a real checkpoint goes through, so every tensor-parallel rank holds its shard of
     the same model and TP=N reproduces TP=1 up to reduction order."""
+    if hasattr(model, "checkpoint_tensors"):
+        # the model family draws tensors under its checkpoint's names; they go through its own placement
+        params = dict(model.named_parameters())
+        for name, t in model.checkpoint_tensors(seed).items():
+            model.load_checkpoint_tensor(params, name, t)
+        return
     dev = next(model.parameters()).device
     g = torch.Generator(device=dev).manual_seed(seed)
     params = dict(model.named_parameters())
