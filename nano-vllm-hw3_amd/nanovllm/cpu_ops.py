@@ -110,7 +110,7 @@ def canon_conv(h, w, state, run, ctx):
         if e <= a:
             continue
         slot, pos0 = int(ctx.seq_slot[b]), int(ctx.seq_pos0[b])
-        prev = state[slot, run].float().clone()                     # [taps-1, W]: inputs at pos0-(taps-1) .. pos0-1
+        prev = state[slot, run][:taps - 1].float().clone()                     # [taps-1, W]: inputs at pos0-(taps-1) .. pos0-1
         for k in range(taps - 1):
             if pos0 - (taps - 1) + k < 0:
                 prev[k] = 0

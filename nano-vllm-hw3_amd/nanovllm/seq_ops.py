@@ -100,7 +100,7 @@ def latent_norm_store(x, w, eps, cache, slot_mapping):
                                             cache.data_ptr(), slot_mapping.data_ptr(), T, R, _dev(x)))
 
 
-USE_TILES = False      # bf16 latent attention on the matrix cores where the shape allows (tests compare both forms)
+USE_TILES = True       # bf16 latent attention on the matrix cores where the shape allows (tests compare both forms)
 
 
 def latent_attention(q, cache, ctx: StepContext, scale, force_rows=False):

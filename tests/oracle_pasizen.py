@@ -4,8 +4,6 @@ sequences at once, no cache, no batching.  Test infrastructure only; it shares n
 Notation.  T tokens, W model width, S residual streams.  Weights are a dict name -> tensor with the checkpoint's
 names ('l3.mix.q', 'l3.mlp.e0.gate', ...); linear weights are [out, in].
 """
-import math
-
 import torch
 
 
@@ -55,10 +53,6 @@ def latent_attention(h, W, p, m, eps):
             a = torch.softmax(s, 0)
             out[i, hh] = a @ v[: i + 1, hh]
     return out.reshape(T, H * V) @ W[p + "o"].T
-
-
-def gelu_tanh(z):
-    return 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))
 
 
 def poly_norm(z, coef, eps):
@@ -147,3 +141,17 @@ def forward(cfg, W, tokens, return_layers=False):
     x = rms_norm(xs.sum(0), W["final.norm"], eps)
     logits = x @ W["head"].T
     return (logits, torch.stack(trace)) if return_layers else logits
+
+
+def absorbed_attention(qa, c, positions, scale):
+    """The attention sum with the key up-projection folded into the query: qa [T, H, R], latents c [N, R] (position j
+    in row j), positions [T] -> o [T, H, R] with o[t, h] = sum_{j <= positions[t]} softmax_j(scale * qa[t, h] . c_j) c_j.
+    (latent_attention above equals W_o applied to W_uv,h o[t, h] with qa[t, h] = W_uk,h^T q[t, h].)"""
+    T, H, R = qa.shape
+    o = torch.zeros(T, H, R)
+    for t in range(T):
+        n = int(positions[t]) + 1
+        for h in range(H):
+            a = torch.softmax((c[:n] @ qa[t, h]) * scale, 0)
+            o[t, h] = a @ c[:n]
+    return o
