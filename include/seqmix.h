@@ -109,6 +109,14 @@ int sm_moe_pairs_gate_up(int dtype, const void* h, const int32_t* idx, const voi
 int sm_moe_pairs_down(int dtype, const void* act, const int32_t* idx, const float* wts, const void* w_down,
                       const void* shared, void* y, int64_t T, int top, int W, int F, void* stream);
 
+/* The same sum for many tokens on the matrix cores (bf16, W % 8 == 0, F % 8 == 0): pairs are grouped by expert into
+ * tiles of 32 rows.  Scratch (caller-owned): n = sm_moe_grouped_tiles(T, top, E) tiles; row_pair int32 [32 n],
+ * tile_expert int32 [n], pair_row int32 [T * top], act bf16 [32 n, F], prod bf16 [32 n, W]. */
+int sm_moe_grouped_tiles(int64_t T, int top, int E);
+int sm_moe_grouped(const void* h, const int32_t* idx, const float* wts, const void* w_gu, const void* w_down,
+                   const void* shared, float limit, float alpha, void* y, int64_t T, int top, int E, int W, int F,
+                   int32_t* row_pair, int32_t* tile_expert, int32_t* pair_row, void* act, void* prod, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

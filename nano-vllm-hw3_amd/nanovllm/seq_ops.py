@@ -174,15 +174,31 @@ def moe_route(h, router_w, top, groups=1, keep=1):
     return idx, wts
 
 
-def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702, shared=None):
+GROUPED_MIN_PAIRS = 128      # from this many (token, expert) pairs on, bf16 experts run grouped on the matrix cores
+
+
+def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702, shared=None, form=None):
     """y[t] = sum_k wts[t, k] * expert_{idx[t, k]}(h[t]) (+ shared[t]); w_gu [E, 2F, W] (gate rows then up rows),
-    w_down [E, W, F]; an expert is a clamped GLU between its two products."""
+    w_down [E, W, F]; an expert is a clamped GLU between its two products.  ``form``: "pairs" | "grouped" to force one."""
     if not h.is_cuda:
         return cpu_ops.moe_experts(h, idx, wts, w_gu, w_down, limit, alpha, shared)
     SM.require_cuda(h, w_gu.dtype, "h")
     T, W = h.shape
     top, F = idx.shape[1], w_down.shape[2]
     lib, code = SM.load(), SM.dtype_code(h.dtype)
+    can_group = h.dtype == torch.bfloat16 and W % 8 == 0 and F % 8 == 0
+    if form == "grouped" or (form is None and can_group and T * top >= GROUPED_MIN_PAIRS):
+        assert can_group
+        E = w_gu.shape[0]
+        n = lib.sm_moe_grouped_tiles(T, top, E)
+        ints = torch.empty(32 * n + n + T * top, dtype=torch.int32, device=h.device)
+        act = torch.empty((32 * n, F), dtype=h.dtype, device=h.device)
+        prod = torch.empty((32 * n, W), dtype=h.dtype, device=h.device)
+        y = torch.empty_like(h)
+        SM.check(lib.sm_moe_grouped(h.data_ptr(), idx.data_ptr(), wts.data_ptr(), w_gu.data_ptr(), w_down.data_ptr(),
+                                    SM.ptr(shared), limit, alpha, y.data_ptr(), T, top, E, W, F, ints.data_ptr(),
+                                    ints[32 * n:].data_ptr(), ints[33 * n:].data_ptr(), act.data_ptr(), prod.data_ptr(), _dev(h)))
+        return y
     act = torch.empty((T * top, F), dtype=h.dtype, device=h.device)
     y = torch.empty_like(h)
     SM.check(lib.sm_moe_pairs_gate_up(code, h.data_ptr(), idx.data_ptr(), w_gu.data_ptr(), limit, alpha, act.data_ptr(), T, top,

@@ -269,6 +269,31 @@ def test_moe_route_and_experts(device, dtype, E, top, groups, keep):
     y = seq_ops.moe_experts(h.to(device, dtype), idx_ref.int().to(device), w_ref.to(device), w_gu.to(device, dtype),
                             w_down.to(device, dtype), 0.7)
     assert torch.allclose(y.float().cpu(), ref, **tol(dtype, 6))
+    if device == "cuda":                        # both forms of the expert products, whatever the dispatcher picks by size
+        forms = ["pairs"] + (["grouped"] if dtype == torch.bfloat16 else [])
+        for form in forms:
+            for sh in (None, shared):
+                y = seq_ops.moe_experts(h.to(device, dtype), idx_ref.int().to(device), w_ref.to(device), w_gu.to(device, dtype),
+                                        w_down.to(device, dtype), 0.7, shared=None if sh is None else sh.to(device, dtype), form=form)
+                assert torch.allclose(y.float().cpu(), ref + (0 if sh is None else sh), **tol(dtype, 6)), form
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,W,F,E,top", [(300, 200, 72, 7, 3), (1, 64, 8, 3, 2), (1000, 256, 384, 16, 4), (65, 72, 40, 40, 1)])
+def test_moe_grouped_equals_pairs(T, W, F, E, top):
+    """Grouped expert products on the matrix cores against the pair-by-pair form: widths and expert sizes that are no
+    multiples of the 64-k step or the 128-column tile, experts without any token, one token, more experts than pairs."""
+    g = gen(T + W)
+    h = rnd(g, T, W).cuda().bfloat16()
+    idx = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(T)]).int()
+    if E > 4:
+        idx[idx == 2] = 3 if top == 1 else idx[idx == 2]            # (top 1: expert 2 gets no token at all)
+    wts = torch.rand(T, top, generator=g)
+    w_gu, w_down, shared = rnd(g, E, 2 * F, W, s=W ** -0.5).cuda().bfloat16(), rnd(g, E, W, F, s=F ** -0.5).cuda().bfloat16(), rnd(g, T, W).cuda().bfloat16()
+    a = seq_ops.moe_experts(h, idx.cuda(), wts.cuda(), w_gu, w_down, 1.2, shared=shared, form="pairs").float()
+    b = seq_ops.moe_experts(h, idx.cuda(), wts.cuda(), w_gu, w_down, 1.2, shared=shared, form="grouped").float()
+    assert torch.allclose(a, b, atol=3e-2, rtol=2e-2)
+    assert (a - b).abs().mean() < 2e-3
 
 
 def test_oracle_absorbed_form_is_the_explicit_one():
