@@ -117,6 +117,13 @@ int sm_moe_grouped(const void* h, const int32_t* idx, const float* wts, const vo
                    const void* shared, float limit, float alpha, void* y, int64_t T, int top, int E, int W, int F,
                    int32_t* row_pair, int32_t* tile_expert, int32_t* pair_row, void* act, void* prod, void* stream);
 
+/* The two ends of sm_moe_grouped on their own (bf16): the grouping (same scratch layout) and the weighted sum of a token's
+ * per-pair products prod [32 n, W] (+ shared).  Between them the caller may run the expert products itself. */
+int sm_moe_align(const int32_t* idx, int64_t T, int top, int E, int32_t* row_pair, int32_t* tile_expert, int32_t* pair_row,
+                 void* stream);
+int sm_moe_combine(const void* prod, const int32_t* pair_row, const float* wts, const void* shared, void* y, int64_t T, int top,
+                   int W, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -6,24 +6,35 @@ namespace sm {
 
 constexpr int kMaxExperts = 1024, kMaxTop = 32;
 
+constexpr int kRouteTokens = 8;      // tokens per workgroup: every router row read serves all of them
+
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, const float* __restrict__ router_w,
-                                                        int32_t* __restrict__ idx, float* __restrict__ wts, int W, int E, int top,
-                                                        int groups, int keep) {
-    extern __shared__ float z[];                 // E scores, then `groups` group scores
-    const int64_t t = blockIdx.x;
+                                                        int32_t* __restrict__ idx, float* __restrict__ wts, int64_t T_all, int W,
+                                                        int E, int top, int groups, int keep) {
+    extern __shared__ float z_all[];             // per token: E scores, then `groups` group scores
+    const int64_t t0 = (int64_t)blockIdx.x * kRouteTokens;
+    const int nt = (int)min((int64_t)kRouteTokens, T_all - t0);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const T* hr = h + (size_t)t * W;
     for (int e = wave; e < E; e += 4) {
         const float* wr = router_w + (size_t)e * W;
-        float d = 0.f;
-        for (int c = lane; c < W; c += 64) d += to_f(hr[c]) * wr[c];
-        d = wave_sum(d);
-        if (lane == 0) z[e] = d;
+        float d[kRouteTokens];
+        for (int i = 0; i < kRouteTokens; ++i) d[i] = 0.f;
+        for (int c = lane; c < W; c += 64) {
+            const float wv = wr[c];
+            for (int i = 0; i < kRouteTokens; ++i)
+                if (i < nt) d[i] += to_f(h[(size_t)(t0 + i) * W + c]) * wv;
+        }
+        for (int i = 0; i < kRouteTokens; ++i) {
+            const float s = wave_sum(d[i]);
+            if (lane == 0) z_all[i * (E + groups) + e] = s;
+        }
     }
     __syncthreads();
-    if (threadIdx.x != 0) return;
-    // one thread finishes the token: E is small and the selections are sequential by nature
+    if (threadIdx.x >= nt) return;
+    // one thread finishes a token: E is small and the selections are sequential by nature
+    const int64_t t = t0 + threadIdx.x;
+    float* z = z_all + threadIdx.x * (E + groups);
     float mx = -INFINITY;
     for (int e = 0; e < E; ++e) mx = fmaxf(mx, z[e]);
     float sum = 0.f;
@@ -148,8 +159,9 @@ extern "C" int sm_moe_route(int dtype, const void* h, const float* router_w, int
     }
     if (T == 0) return SM_OK;
     SM_DISPATCH(dtype, "sm_moe_route",
-                hipLaunchKernelGGL(moe_route_kernel<DT>, dim3((unsigned)T), dim3(256), (size_t)(E + groups) * 4, as_stream(stream),
-                                   (const DT*)h, router_w, idx, wts, W, E, top, groups, keep));
+                hipLaunchKernelGGL(moe_route_kernel<DT>, dim3((unsigned)((T + kRouteTokens - 1) / kRouteTokens)), dim3(256),
+                                   (size_t)kRouteTokens * (E + groups) * 4, as_stream(stream), (const DT*)h, router_w, idx, wts, T, W, E,
+                                   top, groups, keep));
     SM_CHECK_LAUNCH("sm_moe_route");
     return SM_OK;
 }

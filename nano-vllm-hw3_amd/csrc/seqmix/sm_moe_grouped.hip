@@ -161,3 +161,31 @@ extern "C" int sm_moe_grouped(const void* h, const int32_t* idx, const float* wt
     SM_CHECK_LAUNCH("sm_moe_grouped (combine)");
     return SM_OK;
 }
+
+// The grouping and the final sum on their own, for callers that run the expert products themselves (the engine gives
+// large groups to the vendor GEMM, one call per expert on the rows sm_moe_align put together).
+extern "C" int sm_moe_align(const int32_t* idx, int64_t T, int top, int E, int32_t* row_pair, int32_t* tile_expert,
+                            int32_t* pair_row, void* stream) {
+    if (T < 0 || top < 1 || E < 1 || E > 4096 || (T > 0 && (!idx || !row_pair || !tile_expert || !pair_row))) {
+        set_error("sm_moe_align: bad argument");
+        return SM_EINVAL;
+    }
+    if (T == 0) return SM_OK;
+    hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), (size_t)3 * E * sizeof(int), as_stream(stream), idx, (int)(T * top), E,
+                       sm_moe_grouped_tiles(T, top, E), row_pair, tile_expert, pair_row);
+    SM_CHECK_LAUNCH("sm_moe_align");
+    return SM_OK;
+}
+
+extern "C" int sm_moe_combine(const void* prod, const int32_t* pair_row, const float* wts, const void* shared, void* y, int64_t T,
+                              int top, int W, void* stream) {
+    if (T < 0 || top < 1 || W < 1 || (T > 0 && (!prod || !pair_row || !wts || !y))) {
+        set_error("sm_moe_combine: bad argument");
+        return SM_EINVAL;
+    }
+    if (T == 0) return SM_OK;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)T), dim3(256), 0, as_stream(stream), (const unsigned short*)prod, pair_row,
+                       wts, (const unsigned short*)shared, (unsigned short*)y, top, W);
+    SM_CHECK_LAUNCH("sm_moe_combine");
+    return SM_OK;
+}

@@ -29,7 +29,7 @@ __global__ void embed_streams_kernel(const int64_t* __restrict__ ids, const int3
 
 constexpr int kMaxStreams = 8;
 
-template <typename T>
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void stream_step_kernel(float* __restrict__ X, const T* __restrict__ y,
                                                           const float* __restrict__ mix, const float* __restrict__ out,
                                                           const float* __restrict__ w_in, const T* __restrict__ norm_w,
@@ -47,25 +47,43 @@ __global__ __launch_bounds__(256) void stream_step_kernel(float* __restrict__ X,
     __syncthreads();
     float* x = X + (size_t)t * S * W;
     float ss = 0.f;
-    for (int c = threadIdx.x; c < W; c += blockDim.x) {
-        float old[kMaxStreams];
-        for (int s = 0; s < S; ++s) old[s] = x[(size_t)s * W + c];
-        float u = 0.f;
+    // VEC channels per thread (VEC = 4: 16-byte accesses to the f32 streams)
+    for (int c = threadIdx.x * VEC; c < W; c += blockDim.x * VEC) {
+        float old[kMaxStreams][VEC];
+        for (int s = 0; s < S; ++s) {
+            if (VEC == 4) {
+                const float4 v = *(const float4*)(x + (size_t)s * W + c);
+                old[s][0] = v.x; old[s][1] = v.y; old[s][2] = v.z; old[s][VEC - 1] = v.w;
+            } else {
+                old[s][0] = x[(size_t)s * W + c];
+            }
+        }
+        float u[VEC];
+        for (int e = 0; e < VEC; ++e) u[e] = 0.f;
         if (wr) {
-            const float yv = to_f(y[(size_t)t * W + c]);
+            float yv[VEC];
+            for (int e = 0; e < VEC; ++e) yv[e] = to_f(y[(size_t)t * W + c + e]);
             for (int r = 0; r < S; ++r) {
-                float acc = 0.f;
-                for (int s = 0; s < S; ++s) acc += p_mix[s * S + r] * old[s];
-                acc += p_out[r] * yv;
-                x[(size_t)r * W + c] = acc;
-                if (rd) u += p_in[r] * acc;
+                float acc[VEC];
+                for (int e = 0; e < VEC; ++e) {
+                    float a = 0.f;
+                    for (int s = 0; s < S; ++s) a += p_mix[s * S + r] * old[s][e];
+                    a += p_out[r] * yv[e];
+                    acc[e] = a;
+                    if (rd) u[e] += p_in[r] * a;
+                }
+                if (VEC == 4) *(float4*)(x + (size_t)r * W + c) = make_float4(acc[0], acc[1], acc[2], acc[VEC - 1]);
+                else x[(size_t)r * W + c] = acc[0];
             }
         } else if (rd) {
-            for (int s = 0; s < S; ++s) u += p_in[s] * old[s];
+            for (int s = 0; s < S; ++s)
+                for (int e = 0; e < VEC; ++e) u[e] += p_in[s] * old[s][e];
         }
         if (rd) {
-            u_lds[c] = u;
-            ss += u * u;
+            for (int e = 0; e < VEC; ++e) {
+                u_lds[c + e] = u[e];
+                ss += u[e] * u[e];
+            }
         }
     }
     if (!rd) return;
@@ -106,8 +124,12 @@ extern "C" int sm_stream_step(int dtype, float* X, const void* y, const float* m
     if ((size_t)W * 4 > 60000) { set_error("sm_stream_step: width %d too large", W); return SM_ESHAPE; }
     if (T == 0 || (!y && !h_out)) return SM_OK;
     SM_DISPATCH(dtype, "sm_stream_step",
-                hipLaunchKernelGGL(stream_step_kernel<DT>, dim3((unsigned)T), dim3(256), (size_t)W * 4, as_stream(stream), X,
-                                   (const DT*)y, mix, out, w_in, (const DT*)norm_w, eps, (DT*)h_out, S, W));
+                if (W % 4 == 0)
+                    hipLaunchKernelGGL((stream_step_kernel<DT, 4>), dim3((unsigned)T), dim3(256), (size_t)W * 4, as_stream(stream), X,
+                                       (const DT*)y, mix, out, w_in, (const DT*)norm_w, eps, (DT*)h_out, S, W);
+                else
+                    hipLaunchKernelGGL((stream_step_kernel<DT, 1>), dim3((unsigned)T), dim3(256), (size_t)W * 4, as_stream(stream), X,
+                                       (const DT*)y, mix, out, w_in, (const DT*)norm_w, eps, (DT*)h_out, S, W));
     SM_CHECK_LAUNCH("sm_stream_step");
     return SM_OK;
 }

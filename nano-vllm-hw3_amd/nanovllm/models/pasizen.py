@@ -144,12 +144,13 @@ class PasizenForCausalLM(nn.Module):
 
     def checkpoint_tensors(self, seed=0, std=0.05):
         """Random tensors with the checkpoint's names and shapes (benchmarks and tests without a checkpoint), drawn in
-        a fixed order from one seeded generator on the CPU."""
-        cfg, g = self.cfg, torch.Generator().manual_seed(seed)
+        a fixed order from one seeded generator on the model's device."""
+        cfg, dev = self.cfg, self.embed.device
+        g = torch.Generator(device=dev).manual_seed(seed)
         W, S = cfg.hidden_size, cfg.streams
 
         def rnd(*shape, s=std):
-            return torch.randn(*shape, generator=g) * s
+            return torch.randn(*shape, generator=g, device=dev, dtype=torch.float32) * s
         t = {"embed": rnd(cfg.vocab_size, W, s=1.0), "final.norm": 1 + rnd(W), "head": rnd(cfg.vocab_size, W, s=W ** -0.5)}
         if cfg.learned_positions:
             t["pos"] = rnd(cfg.max_position_embeddings, W, s=0.3)
@@ -165,14 +166,14 @@ class PasizenForCausalLM(nn.Module):
             if cfg.learned_streams:
                 for q in ports:
                     t.update({f"{p}{q}.in": 1.0 / S + rnd(S, s=0.1), f"{p}{q}.out": 1 + rnd(S, s=0.1),
-                              f"{p}{q}.mix": torch.eye(S) + rnd(S, S, s=0.1)})
+                              f"{p}{q}.mix": torch.eye(S, device=dev) + rnd(S, S, s=0.1)})
             mlp = spec.get("mlp")
             if mlp is None:
                 continue
             t[p + "norm2"] = 1 + rnd(W)
             if mlp["kind"] == "dense":
                 t.update({p + "mlp.up": rnd(mlp["ff"], W, s=W ** -0.5), p + "mlp.down": rnd(W, mlp["ff"], s=mlp["ff"] ** -0.5),
-                          p + "mlp.act": torch.tensor([0.6, 0.3, 0.1, 0.05]) + rnd(4, s=0.05)})
+                          p + "mlp.act": torch.tensor([0.6, 0.3, 0.1, 0.05], device=dev) + rnd(4, s=0.05)})
                 continue
             ff = mlp["expert"]["ff"]
             t[p + "mlp.router"] = rnd(mlp["router"]["experts"], W, s=2 * W ** -0.5)

@@ -1,0 +1,249 @@
+"""Throughput of the Pasizen family beside the Qwen3 decoder at equal size (random weights, bf16, one GPU), and the
+time of every libseqmix kernel beside the like kernel of the Qwen3 path with both against their rooflines.
+Used by ``bench.py --families``; prints one JSON object."""
+import json
+import os
+import tempfile
+import time
+
+import torch
+
+HBM_GBPS, MFMA_TFLOPS = 8000.0, 2500.0        # MI355X: HBM3E peak, dense bf16 matrix peak
+
+SIZES = {                                      # name -> (width, heads, ff, layers, latent rank)
+    "w1024": (1024, 16, 3072, 4, 128),
+    "w2048": (2048, 16, 6144, 4, 256),
+    "w4096": (4096, 32, 12288, 2, 256),
+}
+VOCAB = 32768
+
+
+def qwen3_config(width, heads, ff, layers):
+    return dict(architectures=["Qwen3ForCausalLM"], hidden_size=width, num_hidden_layers=layers, num_attention_heads=heads,
+                num_key_value_heads=max(1, heads // 2), head_dim=128, intermediate_size=ff, vocab_size=VOCAB, rms_norm_eps=1e-6,
+                rope_theta=1e6, max_position_embeddings=8192, tie_word_embeddings=False, attention_bias=False,
+                hidden_act="silu", torch_dtype="bfloat16")
+
+
+def pasizen_config(width, heads, ff, layers, rank):
+    """Dense (PolyNorm) and routed layers alternate; 16 experts of ff/4 with 4 chosen + one shared: the active
+    feed-forward width of a routed layer is that of the dense one."""
+    mixer = dict(heads=heads, dim=128, vdim=128, kv_rank=rank, scale=128 ** -0.5)
+    moe = dict(kind="moe", expert=dict(ff=ff // 4, limit=7.0),
+               router=dict(experts=16, top=4, groups=dict(count=4, keep=2)), shared=dict(ff=ff // 4, limit=7.0))
+    return dict(architecture="Pasizen", vocab=VOCAB, width=width, max_positions=8192, norm=dict(eps=1e-5), streams=4,
+                canon=dict(taps=4),
+                layers=[dict(type="latent_attention", mixer=mixer, mlp=dict(kind="dense", ff=ff) if i % 2 == 0 else moe)
+                        for i in range(layers)])
+
+
+def _model_dir(cfg):
+    d = tempfile.mkdtemp(prefix="family_bench_")
+    with open(os.path.join(d, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    return d
+
+
+def _timed(fn, reps):
+    fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / reps
+
+
+def engine_throughput(family, size, prefill_seqs=8, prefill_len=1024, decode_seqs=64, decode_ctx=1024, reps=5):
+    """tokens/s of one prefill step (prefill_seqs x prefill_len tokens) and of one decode step (decode_seqs sequences
+    with decode_ctx cached tokens) through the engine's own step function."""
+    from nanovllm import LLM
+    from nanovllm.engine.sequence import ACTIVE, Sequence
+    width, heads, ff, layers, rank = SIZES[size]
+    cfg = pasizen_config(width, heads, ff, layers, rank) if family == "pasizen" else qwen3_config(width, heads, ff, layers)
+    llm = LLM(_model_dir(cfg), load_format="dummy", enforce_eager=family == "pasizen", max_model_len=2048,
+              max_num_seqs=decode_seqs, max_num_batched_tokens=prefill_seqs * prefill_len, gpu_memory_utilization=0.5)
+    g = torch.Generator().manual_seed(0)
+    runner, sch = llm.model_runner, llm.scheduler
+
+    def seqs_of(n, length):
+        out = []
+        for _ in range(n):
+            s = Sequence(torch.randint(0, VOCAB, (length,), generator=g).tolist())
+            s.state = ACTIVE
+            out.append(s)
+        return out
+    res = {}
+    if family == "pasizen":
+        pre = seqs_of(prefill_seqs, prefill_len)
+        for s in pre:
+            assert sch.reserve_portion(s, prefill_len)
+        res["prefill_s"] = _timed(lambda: runner.run_portions([(s, prefill_len) for s in pre]), reps)
+        for s in pre:
+            sch.release(s)
+        dec = seqs_of(decode_seqs, decode_ctx + 1)
+        for s in dec:
+            assert sch.reserve_portion(s, decode_ctx)
+        for i in range(0, decode_seqs, 8):
+            runner.run_portions([(s, decode_ctx) for s in dec[i:i + 8]])
+        for s in dec:
+            s.num_computed = decode_ctx
+            assert sch.reserve_portion(s, 1)
+        res["decode_s"] = _timed(lambda: runner.run_portions([(s, 1) for s in dec]), reps * 4)
+    else:
+        pre = seqs_of(prefill_seqs, prefill_len)
+        for s in pre:
+            sch.block_manager.allocate(s)
+        res["prefill_s"] = _timed(lambda: runner.run(pre, True), reps)
+        for s in pre:
+            sch.block_manager.deallocate(s)
+        dec = seqs_of(decode_seqs, decode_ctx + 1)
+        for s in dec:
+            sch.block_manager.allocate(s)
+        res["decode_s"] = _timed(lambda: runner.run(dec, False), reps * 4)            # hipGraph replay
+        runner.enforce_eager = True
+        res["decode_eager_s"] = _timed(lambda: runner.run(dec, False), reps * 4)
+    out = dict(family=family, size=size, layers=layers, prefill_tokens=prefill_seqs * prefill_len,
+               prefill_tok_per_s=round(prefill_seqs * prefill_len / res["prefill_s"]), decode_batch=decode_seqs,
+               decode_ctx=decode_ctx, decode_tok_per_s=round(decode_seqs / res["decode_s"]),
+               decode_ms_per_step=round(res["decode_s"] * 1e3, 3))
+    if "decode_eager_s" in res:
+        out["decode_eager_tok_per_s"] = round(decode_seqs / res["decode_eager_s"])
+    del llm
+    torch.cuda.empty_cache()
+    return out
+
+
+def _event_time(fn, reps=20):
+    fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e-3 / reps
+
+
+def kernel_table(width=2048, heads=16, rank=256, ff=6144, T=8192, seq=1024, B=64, ctx=1024, streams=4, taps=4):
+    """Seconds per launch of every libseqmix kernel at a layer's size, the bound it works against (bytes / HBM peak or
+    flops / matrix peak) and the fraction of that bound it reaches; beside each the like kernel of the Qwen3 path."""
+    from nanovllm import ops, seq_ops
+    dev, bf = "cuda", torch.bfloat16
+    rows = []
+
+    def add(name, like, sec, bytes_=0, flops=0):
+        bound = max(bytes_ / (HBM_GBPS * 1e9), flops / (MFMA_TFLOPS * 1e12))
+        rows.append(dict(kernel=name, like=like, us=round(sec * 1e6, 1), bound_us=round(bound * 1e6, 1),
+                         of_roofline=round(bound / sec, 3), bound="flops" if flops / (MFMA_TFLOPS * 1e12) > bytes_ / (HBM_GBPS * 1e9) else "bytes"))
+    r = lambda *s: torch.randn(*s, device=dev).to(bf)  # noqa: E731
+    nseq = T // seq
+    # ---- step contexts: a prefill of nseq sequences, a decode of B sequences
+    bs = 64
+
+    def context(portions):
+        tables, nxt = [], 0
+        for p0, n in portions:
+            nb = (p0 + n + bs - 1) // bs
+            tables.append(list(range(nxt, nxt + nb)))
+            nxt += nb
+        import numpy as np
+        tok_seq = np.concatenate([np.full(n, b) for b, (_, n) in enumerate(portions)])
+        tok_pos = np.concatenate([np.arange(p0, p0 + n) for p0, n in portions])
+        slot = np.concatenate([np.asarray(tables[b])[np.arange(p0, p0 + n) // bs] * bs + np.arange(p0, p0 + n) % bs
+                               for b, (p0, n) in enumerate(portions)])
+        mb = max(len(t) for t in tables)
+        bt = np.zeros((len(portions), mb), dtype=np.int32)
+        for b, t in enumerate(tables):
+            bt[b, :len(t)] = t
+        qs = np.concatenate([[0], np.cumsum([n for _, n in portions])])
+        i32 = lambda v: torch.tensor(np.asarray(v), dtype=torch.int32, device=dev)  # noqa: E731
+        return seq_ops.StepContext(tok_seq=i32(tok_seq), tok_pos=i32(tok_pos), qstart=i32(qs), seq_pos0=i32([p for p, _ in portions]),
+                                   ctx_lens=i32([p + n for p, n in portions]), seq_slot=i32(list(range(len(portions)))),
+                                   slot_mapping=i32(slot), block_tables=i32(bt), num_seqs=len(portions), num_tokens=int(qs[-1]),
+                                   max_q=max(n for _, n in portions), block_size=bs), nxt
+    pre, nblk_p = context([(0, seq)] * nseq)
+    dec, nblk_d = context([(ctx - 1, 1)] * B)
+    # ---- residual streams + norm  |  Qwen3: residual add + RMS norm
+    X, y, nw = torch.randn(T, streams, width, device=dev), r(T, width), r(width)
+    mix, out, w_in = torch.randn(streams, streams, device=dev), torch.randn(streams, device=dev), torch.randn(streams, device=dev)
+    add("sm_stream_step (T=%d)" % T, "ql_add_rmsnorm", _event_time(lambda: seq_ops.stream_step(X, y, mix, out, w_in, nw, 1e-5, bf)),
+        bytes_=T * width * (8 * streams + 4))
+    x2, res = r(T, width), r(T, width)
+    add("ql_add_rmsnorm (T=%d)" % T, "-", _event_time(lambda: ops.add_rmsnorm(x2, res, nw, 1e-6)), bytes_=T * width * 8)
+    # ---- short convolution | Qwen3 has none: its elementwise launch (SiLU * mul) is the like kernel
+    h, cw = r(T, width), r(width, taps)
+    state = torch.zeros(nseq, 1, taps - 1, width, device=dev, dtype=bf)
+    add("sm_canon_conv+update (T=%d)" % T, "ql_silu_mul", _event_time(lambda: seq_ops.canon_conv(h, cw, state, 0, pre)), bytes_=T * width * 4)
+    gu = r(T, 2 * ff)
+    add("ql_silu_mul (T=%d)" % T, "-", _event_time(lambda: ops.silu_mul(gu)), bytes_=T * ff * 6)
+    # ---- activations
+    z, coef = r(T, ff), torch.tensor([0.6, 0.3, 0.1, 0.0], device=dev)
+    add("sm_poly_norm (T=%d)" % T, "ql_silu_mul", _event_time(lambda: seq_ops.poly_norm(z, coef, 1e-5)), bytes_=T * ff * 4)
+    add("sm_clamped_glu (T=%d)" % T, "ql_silu_mul", _event_time(lambda: seq_ops.clamped_glu(gu, 7.0)), bytes_=T * ff * 6)
+    # ---- attention, prefill: absorbed queries over the latent | Qwen3: flash attention over K/V of head_dim 128
+    cache = r(max(nblk_p, nblk_d), bs, rank)
+    qa = r(T, heads, rank)
+    pairs = nseq * seq * (seq + 1) / 2 * heads
+    add("sm_latent_attn_tiles (%dx%d, H=%d, R=%d)" % (nseq, seq, heads, rank), "ql_attn_prefill",
+        _event_time(lambda: seq_ops.latent_attention(qa, cache, pre, 0.09), 5), flops=pairs * 4 * rank)
+    q, k, v = r(T, heads, 128), r(T, heads // 2, 128), r(T, heads // 2, 128)
+    cu = torch.arange(0, T + 1, seq, dtype=torch.int32, device=dev)
+    add("ql_attn_prefill (%dx%d, H=%d, D=128)" % (nseq, seq, heads), "-", _event_time(lambda: ops.attn_prefill(q, k, v, cu, seq, 0.09), 5),
+        flops=pairs * 4 * 128)
+    # ---- attention, decode
+    qd = r(B, heads, rank)
+    add("sm_latent_attn_decode (B=%d, ctx=%d, R=%d)" % (B, ctx, rank), "ql_paged_attn_decode",
+        _event_time(lambda: seq_ops.latent_attention(qd, cache, dec, 0.09)), bytes_=B * ctx * rank * 2)
+    kc, vc = r(B * ((ctx + 255) // 256), 256, heads // 2, 128), r(B * ((ctx + 255) // 256), 256, heads // 2, 128)
+    nb = (ctx + 255) // 256
+    tables = torch.arange(B * nb, dtype=torch.int32, device=dev).view(B, nb)
+    lens = torch.full((B,), ctx, dtype=torch.int32, device=dev)
+    ops.reserve_attn_workspace(B, heads, heads // 2, 256, nb, dev)
+    qq = r(B, heads, 128)
+    add("ql_paged_attn_decode (B=%d, ctx=%d, Hkv=%d)" % (B, ctx, heads // 2), "-",
+        _event_time(lambda: ops.paged_attn_decode(qq, kc, vc, tables, lens, 0.09)), bytes_=B * ctx * (heads // 2) * 128 * 4)
+    # ---- latent norm + store | Qwen3: q/k norm + RoPE + K/V store
+    qc = r(T, heads * 128 + rank)
+    add("sm_latent_norm_store (T=%d)" % T, "ql_qknorm_rope_store",
+        _event_time(lambda: seq_ops.latent_norm_store(qc[:, heads * 128:], nw[:rank].contiguous(), 1e-5, cache, pre.slot_mapping)), bytes_=T * rank * 4)
+    # ---- routed experts: many tokens (grouped, matrix cores) and few (pair by pair, weight reads)
+    E, top, F = 16, 4, ff // 4
+    rw = torch.randn(E, width, device=dev)
+    w_gu, w_down = r(E, 2 * F, width), r(E, width, F)
+    add("sm_moe_route (T=%d, E=%d)" % (T, E), "-", _event_time(lambda: seq_ops.moe_route(h, rw, top, 4, 2)), bytes_=T * width * 2)
+    idx, wts = seq_ops.moe_route(h, rw, top, 4, 2)
+    wgu_d, wd_d = r(2 * ff, width), r(width, ff)
+    add("sm_moe_grouped (T=%d, top %d of %d, F=%d)" % (T, top, E, F), "bf16 GEMM of the dense MLP (hipBLASLt)",
+        _event_time(lambda: seq_ops.moe_experts(h, idx, wts, w_gu, w_down, 7.0, form="grouped"), 5), flops=T * top * 6 * width * F)
+    add("routed experts, grouping + hipBLASLt per expert (T=%d)" % T, "bf16 GEMM of the dense MLP (hipBLASLt)",
+        _event_time(lambda: seq_ops.moe_experts(h, idx, wts, w_gu, w_down, 7.0, form="vendor"), 5), flops=T * top * 6 * width * F)
+    hm = h[:512].contiguous()
+    idx_m, wts_m = seq_ops.moe_route(hm, rw, top, 4, 2)
+    add("sm_moe_grouped (T=512)", "bf16 GEMM of the dense MLP (hipBLASLt)",
+        _event_time(lambda: seq_ops.moe_experts(hm, idx_m, wts_m, w_gu, w_down, 7.0, form="grouped"), 5), flops=512 * top * 6 * width * F,
+        bytes_=E * 3 * F * width * 2)
+    add("dense MLP GEMMs, hipBLASLt (T=512)", "-",
+        _event_time(lambda: torch.nn.functional.linear(torch.nn.functional.linear(hm, wgu_d)[:, :ff], wd_d), 5), flops=512 * 6 * width * ff,
+        bytes_=3 * ff * width * 2)
+    add("dense MLP GEMMs, hipBLASLt (T=%d, ff=%d)" % (T, ff), "-",
+        _event_time(lambda: torch.nn.functional.linear(torch.nn.functional.linear(h, wgu_d)[:, :ff], wd_d), 5), flops=T * 6 * width * ff)
+    hd = h[:B].contiguous()
+    idx_d, wts_d = seq_ops.moe_route(hd, rw, top, 4, 2)
+    touched = len(torch.unique(idx_d))
+    add("sm_moe_grouped (T=%d: decode)" % B, "bf16 GEMM of the dense MLP (hipBLASLt)",
+        _event_time(lambda: seq_ops.moe_experts(hd, idx_d, wts_d, w_gu, w_down, 7.0, form="grouped")), bytes_=touched * 3 * F * width * 2)
+    add("dense MLP GEMMs, hipBLASLt (T=%d: decode)" % B, "-",
+        _event_time(lambda: torch.nn.functional.linear(torch.nn.functional.linear(hd, wgu_d)[:, :ff], wd_d)), bytes_=3 * ff * width * 2)
+    return rows
+
+
+def main(sizes=("w1024", "w2048"), kernels=True):
+    out = dict(metric="family comparison", dtype="bf16", data="synthetic (random weights)", throughput=[], kernels=[])
+    for size in sizes:
+        for family in ("pasizen", "qwen3"):
+            out["throughput"].append(engine_throughput(family, size))
+    if kernels:
+        out["kernels"] = kernel_table()
+    return out
