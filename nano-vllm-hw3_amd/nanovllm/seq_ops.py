@@ -174,16 +174,10 @@ def moe_route(h, router_w, top, groups=1, keep=1):
     return idx, wts
 
 
-# bf16 experts run grouped by expert on the matrix cores: the libseqmix kernel up to this many (token, expert) pairs per
-# expert on average, beyond it the vendor GEMM, one call per expert on the grouped rows (the group sizes are read back
-# to the host for that: one small copy per routed layer of a large step)
-VENDOR_MIN_ROWS_PER_EXPERT = 256
-
-
 def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702, shared=None, form=None):
     """y[t] = sum_k wts[t, k] * expert_{idx[t, k]}(h[t]) (+ shared[t]); w_gu [E, 2F, W] (gate rows then up rows),
-    w_down [E, W, F]; an expert is a clamped GLU between its two products.  ``form``: "pairs" | "grouped" | "vendor"
-    forces one; by default float32 runs pair by pair and bf16 grouped."""
+    w_down [E, W, F]; an expert is a clamped GLU between its two products.  ``form``: "pairs" | "grouped" forces
+    one; by default float32 runs pair by pair and bf16 grouped by expert on the matrix cores."""
     if not h.is_cuda:
         return cpu_ops.moe_experts(h, idx, wts, w_gu, w_down, limit, alpha, shared)
     SM.require_cuda(h, w_gu.dtype, "h")
@@ -193,40 +187,20 @@ def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702, shared=None, form
     lib, code = SM.load(), SM.dtype_code(h.dtype)
     can_group = h.dtype == torch.bfloat16 and W % 8 == 0 and F % 8 == 0
     if form is None:
-        form = "pairs" if not can_group else ("vendor" if T * top >= VENDOR_MIN_ROWS_PER_EXPERT * E and
-                                              not torch.cuda.is_current_stream_capturing() else "grouped")
-    if form in ("grouped", "vendor"):
+        form = "grouped" if can_group else "pairs"
+    if form == "grouped":
         assert can_group
         n = lib.sm_moe_grouped_tiles(T, top, E)
         ints = torch.empty(32 * n + n + T * top, dtype=torch.int32, device=h.device)
         row_pair, tile_expert, pair_row = ints[:32 * n], ints[32 * n:33 * n], ints[33 * n:]
         y = torch.empty_like(h)
         prod = torch.empty((32 * n, W), dtype=h.dtype, device=h.device)
-        if form == "grouped":
-            act = torch.empty((32 * n, F), dtype=h.dtype, device=h.device)
-            SM.check(lib.sm_moe_grouped(h.data_ptr(), idx.data_ptr(), wts.data_ptr(), w_gu.data_ptr(), w_down.data_ptr(),
-                                        SM.ptr(shared), limit, alpha, y.data_ptr(), T, top, E, W, F, row_pair.data_ptr(),
-                                        tile_expert.data_ptr(), pair_row.data_ptr(), act.data_ptr(), prod.data_ptr(), _dev(h)))
-            return y
-        SM.check(lib.sm_moe_align(idx.data_ptr(), T, top, E, row_pair.data_ptr(), tile_expert.data_ptr(), pair_row.data_ptr(), _dev(h)))
-        counts = torch.bincount(tile_expert[tile_expert >= 0], minlength=E).tolist()       # tiles of 32 rows per expert
-        hs = h.index_select(0, row_pair.clamp(min=0) // top)                                 # rows grouped by expert
-        gu = torch.empty((32 * n, 2 * F), dtype=h.dtype, device=h.device)
-        a = 0
-        for e, c in enumerate(counts):
-            if c:
-                torch.mm(hs[a:a + 32 * c], w_gu[e].t(), out=gu[a:a + 32 * c])
-            a += 32 * c
-        if a < 32 * n:
-            gu[a:].zero_()
-        act = clamped_glu(gu, limit, alpha)
-        a = 0
-        for e, c in enumerate(counts):
-            if c:
-                torch.mm(act[a:a + 32 * c], w_down[e].t(), out=prod[a:a + 32 * c])
-            a += 32 * c
-        SM.check(lib.sm_moe_combine(prod.data_ptr(), pair_row.data_ptr(), wts.data_ptr(), SM.ptr(shared), y.data_ptr(), T, top, W, _dev(h)))
+        act = torch.empty((32 * n, F), dtype=h.dtype, device=h.device)
+        SM.check(lib.sm_moe_grouped(h.data_ptr(), idx.data_ptr(), wts.data_ptr(), w_gu.data_ptr(), w_down.data_ptr(),
+                                    SM.ptr(shared), limit, alpha, y.data_ptr(), T, top, E, W, F, row_pair.data_ptr(),
+                                    tile_expert.data_ptr(), pair_row.data_ptr(), act.data_ptr(), prod.data_ptr(), _dev(h)))
         return y
+    assert form == "pairs", form
     act = torch.empty((T * top, F), dtype=h.dtype, device=h.device)
     y = torch.empty_like(h)
     SM.check(lib.sm_moe_pairs_gate_up(code, h.data_ptr(), idx.data_ptr(), w_gu.data_ptr(), limit, alpha, act.data_ptr(), T, top,
