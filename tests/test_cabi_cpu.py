@@ -96,3 +96,38 @@ def test_ops_refuse_cpu_tensors():
         NQ.per_row_quant(x, torch.int8)
     with pytest.raises(Q.QLinearError):
         NQ.per_group_quant(x, 64, torch.int8)
+
+
+# ---- libseqmix (include/seqmix.h) --------------------------------------------------------------------------------------
+SEQMIX_HEADER = os.path.join(ROOT, "include", "seqmix.h")
+
+
+def seqmix_declared():
+    src = re.sub(r"/\*.*?\*/", "", open(SEQMIX_HEADER).read(), flags=re.S)
+    return sorted(set(re.findall(r"\b(sm_[a-z0-9_]+)\s*\(", src)))
+
+
+def test_seqmix_binding_covers_header_and_library_exports_it():
+    from nanovllm import _seqmix as SM
+    SM.build_if_missing()
+    lib = ctypes.CDLL(SM.LIB_PATH)
+    names = seqmix_declared()
+    assert sorted(SM.SIGNATURES) == names
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in seqmix.h but not exported"
+    assert SM.load().sm_version() >= 1
+
+
+def test_seqmix_argument_validation_needs_no_gpu():
+    from nanovllm import _seqmix as SM
+    lib = SM.load()
+    one = ctypes.c_void_p(16)   # never dereferenced: the calls below are rejected first
+    assert lib.sm_stream_step(7, one, one, one, one, one, one, 1e-5, one, 4, 2, 64, None) == -1          # unknown dtype
+    assert lib.sm_stream_step(1, one, one, one, one, one, one, 1e-5, one, 4, 9, 64, None) == -2          # too many streams
+    assert b"streams" in lib.sm_last_error()
+    assert lib.sm_canon_conv(1, one, one, one, 3, 3, one, one, one, one, one, 4, 64, 4, None) == -1      # run >= runs
+    assert lib.sm_latent_attn_tiles(one, one, one, one, one, one, 0.1, 2, 8, 4, 36, 64, 4, None) == -2   # R % 8
+    assert lib.sm_latent_attn_tiles(one, one, one, one, one, one, 0.1, 2, 8, 4, 64, 48, 4, None) == -2   # block % 64
+    assert lib.sm_latent_attn_decode(one, one, one, one, one, 0.1, 2, 4, 64, 64, 4, 2, one, 16, None) == -3   # workspace
+    assert lib.sm_moe_route(1, one, one, one, one, 4, 64, 8, 3, 4, 1, None) == -2                        # top > keep * E/groups
+    assert lib.sm_moe_grouped(one, one, one, one, one, None, 1.0, 1.7, one, 4, 2, 8, 60, 64, one, one, one, one, one, None) == -2
