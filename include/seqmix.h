@@ -117,6 +117,14 @@ int sm_moe_grouped(const void* h, const int32_t* idx, const float* wts, const vo
                    const void* shared, float limit, float alpha, void* y, int64_t T, int top, int E, int W, int F,
                    int32_t* row_pair, int32_t* tile_expert, int32_t* pair_row, void* act, void* prod, void* stream);
 
+/* sm_moe_grouped with tiles of 128 rows (activations of a tile staged once in LDS, every weight fragment reused by four
+ * row fragments): the form for large groups.  Same arguments; scratch for n = sm_moe_tiles128_count(T, top, E) tiles:
+ * row_pair int32 [128 n], tile_expert int32 [n], pair_row int32 [T * top], act bf16 [128 n, F], prod bf16 [128 n, W]. */
+int sm_moe_tiles128_count(int64_t T, int top, int E);
+int sm_moe_tiles128(const void* h, const int32_t* idx, const float* wts, const void* w_gu, const void* w_down,
+                    const void* shared, float limit, float alpha, void* y, int64_t T, int top, int E, int W, int F,
+                    int32_t* row_pair, int32_t* tile_expert, int32_t* pair_row, void* act, void* prod, void* stream);
+
 /* The two ends of sm_moe_grouped on their own (bf16): the grouping (same scratch layout) and the weighted sum of a token's
  * per-pair products prod [32 n, W] (+ shared).  Between them the caller may run the expert products itself. */
 int sm_moe_align(const int32_t* idx, int64_t T, int top, int E, int32_t* row_pair, int32_t* tile_expert, int32_t* pair_row,

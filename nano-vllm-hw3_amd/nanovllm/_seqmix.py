@@ -33,6 +33,8 @@ SIGNATURES = {
     "sm_moe_pairs_gate_up": (_int, [_int, _vp, _vp, _vp, _f, _f, _vp, _i64, _int, _int, _int, _vp]),
     "sm_moe_pairs_down": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _int, _vp]),
     "sm_moe_grouped_tiles": (_int, [_i64, _int, _int]),
+    "sm_moe_tiles128_count": (_int, [_i64, _int, _int]),
+    "sm_moe_tiles128": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _vp, _i64, _int, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp]),
     "sm_moe_align": (_int, [_vp, _i64, _int, _int, _vp, _vp, _vp, _vp]),
     "sm_moe_combine": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "sm_moe_grouped": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _vp, _i64, _int, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp]),

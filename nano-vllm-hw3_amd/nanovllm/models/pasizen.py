@@ -93,6 +93,7 @@ class PasizenForCausalLM(nn.Module):
         self.head = nn.Parameter(torch.empty(cfg.vocab_size, W), requires_grad=False)
         self.run_order = list(cfg.run_order)
         self.sum_streams = torch.ones(cfg.streams, dtype=torch.float32)
+        self._f32_out = None       # whether the vendor GEMM writes float32 from 16-bit operands for the head's shape
 
     # ------------------------------------------------------------------ checkpoint names
     _SIMPLE = {"norm1": "norm1", "norm2": "norm2", "canon1": "canon.weight", "mix.dkv.norm": "mixer.latent_norm",
@@ -244,6 +245,13 @@ class PasizenForCausalLM(nn.Module):
         """float32 logits of the given rows: products of the stored values, float32 accumulation AND output."""
         if hidden_states.dtype == torch.float32:
             return F.linear(hidden_states, self.head)
-        if hidden_states.is_cuda:
-            return torch.mm(hidden_states, self.head.t(), out_dtype=torch.float32)
+        if hidden_states.is_cuda and self._f32_out is not False:
+            try:
+                out = torch.mm(hidden_states, self.head.t(), out_dtype=torch.float32)
+                self._f32_out = True
+                return out
+            except RuntimeError:
+                if self._f32_out:          # it has worked before: this is another fault
+                    raise
+                self._f32_out = False      # no such GEMM for this shape: the same sums from widened operands
         return F.linear(hidden_states.float(), self.head.float())

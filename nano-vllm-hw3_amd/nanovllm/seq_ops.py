@@ -114,7 +114,7 @@ def latent_attention(q, cache, ctx: StepContext, scale, force_rows=False):
     lib = SM.load()
     bs, mb = cache.shape[1], ctx.block_tables.shape[1]
     tiles_ok = (USE_TILES and not force_rows and q.dtype == torch.bfloat16 and R % 8 == 0 and R <= 256 and bs % 64 == 0)
-    if tiles_ok and ctx.max_q == 1:
+    if tiles_ok and ctx.max_q == 1 and H <= 128:
         splits = decode_splits(ctx.num_seqs, mb * bs)
         ws, n = SM.decode_workspace.get(q.device, lib.sm_latent_decode_workspace_bytes(T, H, R, splits))
         SM.check(lib.sm_latent_attn_decode(q.data_ptr(), cache.data_ptr(), ctx.block_tables.data_ptr(), ctx.ctx_lens.data_ptr(),
@@ -174,10 +174,14 @@ def moe_route(h, router_w, top, groups=1, keep=1):
     return idx, wts
 
 
+TILES128_MIN_ROWS_PER_EXPERT = 64
+
+
 def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702, shared=None, form=None):
     """y[t] = sum_k wts[t, k] * expert_{idx[t, k]}(h[t]) (+ shared[t]); w_gu [E, 2F, W] (gate rows then up rows),
-    w_down [E, W, F]; an expert is a clamped GLU between its two products.  ``form``: "pairs" | "grouped" forces
-    one; by default float32 runs pair by pair and bf16 grouped by expert on the matrix cores."""
+    w_down [E, W, F]; an expert is a clamped GLU between its two products.  ``form``: "pairs" | "grouped" | "tiles128"
+    forces one; by default float32 runs pair by pair and bf16 grouped by expert on the matrix cores, in tiles of 32 rows
+    for small groups (decode) and of 128 rows for large ones (prefill)."""
     if not h.is_cuda:
         return cpu_ops.moe_experts(h, idx, wts, w_gu, w_down, limit, alpha, shared)
     SM.require_cuda(h, w_gu.dtype, "h")
@@ -187,18 +191,21 @@ def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702, shared=None, form
     lib, code = SM.load(), SM.dtype_code(h.dtype)
     can_group = h.dtype == torch.bfloat16 and W % 8 == 0 and F % 8 == 0
     if form is None:
-        form = "grouped" if can_group else "pairs"
-    if form == "grouped":
+        # groups of 64 rows and more on average fill 128-row tiles well enough to pay for their padding
+        form = "pairs" if not can_group else ("tiles128" if T * top >= TILES128_MIN_ROWS_PER_EXPERT * E else "grouped")
+    if form in ("grouped", "tiles128"):
         assert can_group
-        n = lib.sm_moe_grouped_tiles(T, top, E)
-        ints = torch.empty(32 * n + n + T * top, dtype=torch.int32, device=h.device)
-        row_pair, tile_expert, pair_row = ints[:32 * n], ints[32 * n:33 * n], ints[33 * n:]
+        rows = 32 if form == "grouped" else 128
+        n = lib.sm_moe_grouped_tiles(T, top, E) if form == "grouped" else lib.sm_moe_tiles128_count(T, top, E)
+        ints = torch.empty(rows * n + n + T * top, dtype=torch.int32, device=h.device)
+        row_pair, tile_expert, pair_row = ints[:rows * n], ints[rows * n:rows * n + n], ints[rows * n + n:]
         y = torch.empty_like(h)
-        prod = torch.empty((32 * n, W), dtype=h.dtype, device=h.device)
-        act = torch.empty((32 * n, F), dtype=h.dtype, device=h.device)
-        SM.check(lib.sm_moe_grouped(h.data_ptr(), idx.data_ptr(), wts.data_ptr(), w_gu.data_ptr(), w_down.data_ptr(),
+        prod = torch.empty((rows * n, W), dtype=h.dtype, device=h.device)
+        act = torch.empty((rows * n, F), dtype=h.dtype, device=h.device)
+        fn = lib.sm_moe_grouped if form == "grouped" else lib.sm_moe_tiles128
+        SM.check(fn(h.data_ptr(), idx.data_ptr(), wts.data_ptr(), w_gu.data_ptr(), w_down.data_ptr(),
                                     SM.ptr(shared), limit, alpha, y.data_ptr(), T, top, E, W, F, row_pair.data_ptr(),
-                                    tile_expert.data_ptr(), pair_row.data_ptr(), act.data_ptr(), prod.data_ptr(), _dev(h)))
+                    tile_expert.data_ptr(), pair_row.data_ptr(), act.data_ptr(), prod.data_ptr(), _dev(h)))
         return y
     assert form == "pairs", form
     act = torch.empty((T * top, F), dtype=h.dtype, device=h.device)

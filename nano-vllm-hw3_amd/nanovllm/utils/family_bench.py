@@ -217,6 +217,8 @@ def kernel_table(width=2048, heads=16, rank=256, ff=6144, T=8192, seq=1024, B=64
     wgu_d, wd_d = r(2 * ff, width), r(width, ff)
     add("sm_moe_grouped (T=%d, top %d of %d, F=%d)" % (T, top, E, F), "bf16 GEMM of the dense MLP (hipBLASLt)",
         _event_time(lambda: seq_ops.moe_experts(h, idx, wts, w_gu, w_down, 7.0, form="grouped"), 5), flops=T * top * 6 * width * F)
+    add("sm_moe_tiles128 (T=%d, top %d of %d, F=%d)" % (T, top, E, F), "bf16 GEMM of the dense MLP (hipBLASLt)",
+        _event_time(lambda: seq_ops.moe_experts(h, idx, wts, w_gu, w_down, 7.0, form="tiles128"), 5), flops=T * top * 6 * width * F)
     hm = h[:512].contiguous()
     idx_m, wts_m = seq_ops.moe_route(hm, rw, top, 4, 2)
     add("sm_moe_grouped (T=512)", "bf16 GEMM of the dense MLP (hipBLASLt)",

@@ -270,7 +270,7 @@ def test_moe_route_and_experts(device, dtype, E, top, groups, keep):
                             w_down.to(device, dtype), 0.7)
     assert torch.allclose(y.float().cpu(), ref, **tol(dtype, 6))
     if device == "cuda":                        # both forms of the expert products, whatever the dispatcher picks by size
-        forms = ["pairs"] + (["grouped"] if dtype == torch.bfloat16 else [])
+        forms = ["pairs"] + (["grouped", "tiles128"] if dtype == torch.bfloat16 else [])
         for form in forms:
             for sh in (None, shared):
                 y = seq_ops.moe_experts(h.to(device, dtype), idx_ref.int().to(device), w_ref.to(device), w_gu.to(device, dtype),
@@ -294,6 +294,8 @@ def test_moe_grouped_equals_pairs(T, W, F, E, top):
     b = seq_ops.moe_experts(h, idx.cuda(), wts.cuda(), w_gu, w_down, 1.2, shared=shared, form="grouped").float()
     assert torch.allclose(a, b, atol=3e-2, rtol=2e-2)
     assert (a - b).abs().mean() < 2e-3
+    c = seq_ops.moe_experts(h, idx.cuda(), wts.cuda(), w_gu, w_down, 1.2, shared=shared, form="tiles128").float()
+    assert torch.equal(b, c)          # a row's sums do not depend on the tile it sits in: both grouped forms agree exactly
 
 
 def test_oracle_absorbed_form_is_the_explicit_one():
