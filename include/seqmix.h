@@ -110,7 +110,9 @@ int sm_moe_pairs_down(int dtype, const void* act, const int32_t* idx, const floa
                       const void* shared, void* y, int64_t T, int top, int W, int F, void* stream);
 
 /* The same sum for many tokens on the matrix cores (bf16, W % 8 == 0, F % 8 == 0): pairs are grouped by expert into
- * tiles of 32 rows.  Scratch (caller-owned): n = sm_moe_grouped_tiles(T, top, E) tiles; row_pair int32 [32 n],
+ * tiles of 32 rows.  w_gu and w_down are TILED here: blocks of 32 rows x 64 k (4 KB; rows and k zero-padded to whole
+ * blocks) in the order (expert, gate|up, row block, k step); inside a block the 8 values k = 64 step + 32 hi + 8 s .. +8
+ * of row r sit at byte 16 (64 s + 32 hi + r).  Scratch (caller-owned): n = sm_moe_grouped_tiles(T, top, E) tiles; row_pair int32 [32 n],
  * tile_expert int32 [n], pair_row int32 [T * top], act bf16 [32 n, F], prod bf16 [32 n, W]. */
 int sm_moe_grouped_tiles(int64_t T, int top, int E);
 int sm_moe_grouped(const void* h, const int32_t* idx, const float* wts, const void* w_gu, const void* w_down,

@@ -77,24 +77,45 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const unsigned short* 
     const int row = tile * kRowsPerTile + l31;
     const int pair = row_pair[row];
     const unsigned short* ap = GATE_UP ? a + (size_t)(pair < 0 ? 0 : pair / top) * K : a + (size_t)row * K;
-    const int col = min(n0 + l31, N - 1);
-    const unsigned short* bp = w + ((size_t)e * (GATE_UP ? 2 : 1) * N + col) * K;
-    const unsigned short* bp2 = bp + (size_t)N * K;           // the up rows follow the gate rows
+    // weights in the tiled layout of sm_moe_tile_weights: block (expert, 32-row block, 64-k step) = 4 KB, chunk s of
+    // lane L at 16 (64 s + L): a wave's load is one contiguous KB
+    const int nb32 = (N + 31) / 32, ksteps = (K + 63) / 64;
+    const unsigned short* bp = w + (((size_t)e * (GATE_UP ? 2 : 1) * nb32 + n0 / 32) * ksteps) * 2048 + 8 * lane;
+    const unsigned short* bp2 = bp + (size_t)nb32 * ksteps * 2048;      // the up blocks follow the gate blocks
     f32x16 acc = {0}, acc2 = {0};
-    for (int k0 = 0; k0 < K; k0 += 64) {
+    // A ring of three 64-k steps in flight: with a handful of rows per expert (decode) a wave's eight MFMAs per step
+    // hide nothing, so the weight stream has to be kept busy by outstanding loads (3 x 12 KB per wave).  Steps past K
+    // load zeros (both operands), which leave the sums as they are.
+    struct Stage { bf16x8 a[4], b[4], b2[4]; };
+    auto request = [&](Stage& st, int k0) {
         const int kb = k0 + 32 * hi;
-        bf16x8 af[4], bf[4], bf2[4];
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            af[s] = load8(ap, kb + 8 * s, K);
-            bf[s] = load8(bp, kb + 8 * s, K);
-            if (GATE_UP) bf2[s] = load8(bp2, kb + 8 * s, K);
+            st.a[s] = load8(ap, kb + 8 * s, K);
+            // (steps past K: the ring runs up to two steps over; clamp to the last block and let A's zeros cancel it)
+            const size_t boff = (size_t)min(k0 / 64, ksteps - 1) * 2048 + 512 * s;
+            st.b[s] = *(const bf16x8*)(bp + boff);
+            if (GATE_UP) st.b2[s] = *(const bf16x8*)(bp2 + boff);
         }
+    };
+    auto consume = [&](const Stage& st) {
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[s], bf[s], acc, 0, 0, 0);
-            if (GATE_UP) acc2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[s], bf2[s], acc2, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(st.a[s], st.b[s], acc, 0, 0, 0);
+            if (GATE_UP) acc2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(st.a[s], st.b2[s], acc2, 0, 0, 0);
         }
+    };
+    Stage s0, s1, s2;
+    request(s0, 0);
+    request(s1, 64);
+    request(s2, 128);
+    for (int k0 = 0; k0 < K; k0 += 192) {
+        consume(s0);
+        request(s0, k0 + 192);
+        consume(s1);
+        request(s1, k0 + 256);
+        consume(s2);
+        request(s2, k0 + 320);
     }
     if (n0 + l31 >= N) return;
 #pragma unroll

@@ -81,9 +81,10 @@ __global__ __launch_bounds__(256) void moe_tiles128_kernel(const unsigned short*
     const int srow = tid >> 1, shalf = tid & 1;
     const int spair = row_pair[tile * kBigRows + srow];
     const unsigned short* ap = GATE_UP ? a + (size_t)(spair < 0 ? 0 : spair / top) * K : a + ((size_t)tile * kBigRows + srow) * K;
-    const int col = min(n0 + l31, N - 1);
-    const unsigned short* bp = w + ((size_t)e * (GATE_UP ? 2 : 1) * N + col) * K;
-    const unsigned short* bp2 = bp + (size_t)N * K;           // the up rows follow the gate rows
+    // weights in the tiled layout of sm_moe_tile_weights (see sm_moe_grouped.hip): a wave's load is one contiguous KB
+    const int nb32 = (N + 31) / 32, ksteps = (K + 63) / 64;
+    const unsigned short* bp = w + (((size_t)e * (GATE_UP ? 2 : 1) * nb32 + min(n0, N - 1) / 32) * ksteps) * 2048 + 8 * lane;
+    const unsigned short* bp2 = bp + (size_t)nb32 * ksteps * 2048;      // the up blocks follow the gate blocks
     f32x16 acc[4], acc2[4];
 #pragma unroll
     for (int m = 0; m < 4; ++m)
@@ -95,8 +96,9 @@ __global__ __launch_bounds__(256) void moe_tiles128_kernel(const unsigned short*
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             ar[s] = load16(ap, k0 + 32 * shalf + 8 * s, K);
-            bn[s] = load16(bp, k0 + 32 * hi + 8 * s, K);
-            if (GATE_UP) bn2[s] = load16(bp2, k0 + 32 * hi + 8 * s, K);
+            const size_t boff = (size_t)(k0 / 64) * 2048 + 512 * s;
+            bn[s] = *(const i32x4*)(bp + boff);
+            if (GATE_UP) bn2[s] = *(const i32x4*)(bp2 + boff);
         }
     };
     request(0);

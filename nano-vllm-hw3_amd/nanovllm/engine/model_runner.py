@@ -101,10 +101,97 @@ class ModelRunner:
         if cfg.num_kvcache_blocks > 0:            # an explicit pool size (tests, replaying a trace): taken as given
             max_needed = cfg.num_kvcache_blocks
         cfg.num_kvcache_blocks = max(1, min(budget // max(block_bytes, 1), max_needed))
-        self.model.allocate_cache(cfg.num_kvcache_blocks, bs, slots, self.device)
+        # one block and one slot more than the pools hand out: where the padding rows of a captured decode step write
+        self.model.allocate_cache(cfg.num_kvcache_blocks + 1, bs, slots + 1, self.device)
         self._stage_max_bs = 0
         self._stage_rows = []
         self._tok_host = [torch.zeros(0, dtype=torch.int64)]
+        self.portion_graphs = {}
+        if self.on_gpu and not self.enforce_eager:
+            self._capture_portion_graphs()
+
+    # decode-only steps of a portion model replay a hipGraph per batch-size bucket, as the Qwen3 decode steps do
+    def _decode_layout(self, B, mb):
+        sizes = [2 * B, B, B, B, B + 1, B, B, B, B * mb]
+        offs = [0]
+        for n in sizes:
+            offs.append(offs[-1] + n)
+        return offs
+
+    def _capture_portion_graphs(self):
+        from nanovllm import _seqmix, seq_ops
+        cfg, bs = self.config, self.block_size
+        mb = (cfg.max_model_len + bs - 1) // bs
+        self._graph_mb = mb
+        scratch_block, scratch_slot = cfg.num_kvcache_blocks, cfg.max_num_seqs
+        buckets = [b for b in (1, 2, 4, 8, 16, 32, 64, 128, 256) if b < cfg.max_num_seqs] + [min(cfg.max_num_seqs, 256)]
+        pool = None
+        for gb in sorted(set(buckets), reverse=True):
+            offs = self._decode_layout(gb, mb)
+            host = torch.zeros(offs[-1] + 1, dtype=torch.int32, device="cpu", pin_memory=True)
+            hv = host.numpy()
+            # every row starts as a padding row: token 0 at position 0 of a one-token sequence in the scratch block / slot
+            hv[offs[1]:offs[2]] = range(gb)                      # tok_seq
+            hv[offs[3]:offs[4]] = scratch_block * bs             # slot_mapping
+            hv[offs[4]:offs[5]] = range(gb + 1)                  # qstart
+            hv[offs[6]:offs[7]] = 1                              # ctx_lens
+            hv[offs[7]:offs[8]] = scratch_slot                   # seq_slot
+            hv[offs[8]:offs[9]] = scratch_block                  # block tables
+            pad = host.clone()
+            dev = host.to(self.device)
+            v = [dev[offs[i]:offs[i + 1]] for i in range(9)]
+            step = seq_ops.StepContext(tok_seq=v[1], tok_pos=v[2], slot_mapping=v[3], qstart=v[4], seq_pos0=v[5], ctx_lens=v[6],
+                                       seq_slot=v[7], block_tables=v[8].view(gb, mb), num_seqs=gb, num_tokens=gb, max_q=1,
+                                       block_size=bs, qstart_host=list(range(gb + 1)))
+            ids = v[0].view(torch.int64)
+            logits = torch.zeros(gb, cfg.hf_config.vocab_size, dtype=torch.float32, device=self.device)
+
+            def body():
+                logits.copy_(self.model.compute_logits(self.model(ids, v[2])))
+            seq_ops.set_step(step)
+            try:
+                with torch.no_grad():
+                    body()                                       # warm-up: sizes every workspace, settles lazy choices
+                    torch.cuda.synchronize()
+                    g = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(g, pool):
+                        body()
+            finally:
+                seq_ops.set_step(None)
+            if pool is None:
+                pool = g.pool()
+            self.portion_graphs[gb] = dict(graph=g, host=host, pad=pad, dev=dev, offs=offs, logits=logits)
+        torch.cuda.synchronize()
+        _seqmix.decode_workspace.pin(self.device)                # the graphs address it: never freed
+
+    def _replay_decode(self, batch):
+        """A step of single tokens through the captured graph of the smallest bucket that holds it; float32 logits [B, vocab]."""
+        import numpy as np
+        B, bs, mb = len(batch), self.block_size, self._graph_mb
+        gb = min(k for k in self.portion_graphs if k >= B)
+        e = self.portion_graphs[gb]
+        offs, host = e["offs"], e["host"]
+        host.copy_(e["pad"])
+        hv = host.numpy()
+        ids = hv[offs[0]:offs[1]].view(np.int64)
+        tables = hv[offs[8]:offs[9]].reshape(gb, mb)
+        for b, (seq, n) in enumerate(batch):
+            p = seq.num_computed
+            assert n == 1 and p < seq.num_tokens and seq.state_slot >= 0 and len(seq.block_table) * bs > p
+            ids[b] = seq.token_ids[p]
+            hv[offs[2] + b] = p                                   # tok_pos
+            hv[offs[3] + b] = seq.block_table[p // bs] * bs + p % bs
+            hv[offs[5] + b] = p                                   # seq_pos0
+            hv[offs[6] + b] = p + 1                               # ctx_lens
+            hv[offs[7] + b] = seq.state_slot
+            nb = p // bs + 1
+            tables[b, :nb] = seq.block_table[:nb]
+        e["dev"].copy_(host, non_blocking=True)
+        e["graph"].replay()
+        out = e["logits"][:B].clone()
+        # (the pinned mirror is rewritten by the next step: the copy above must have left it)
+        torch.cuda.current_stream().synchronize()
+        return out
 
     def prepare_portions(self, batch):
         """[(sequence, token count)] -> (input ids, positions, StepContext).  Every index the kernels need travels in
@@ -154,6 +241,11 @@ class ModelRunner:
         steps left.  Returns float32 logits of ``rows`` (indices into the step's packed tokens; default: the last token
         of every portion, in batch order)."""
         from nanovllm import seq_ops
+        B = len(batch)
+        if (self.portion_graphs and trace is None and all(n == 1 for _, n in batch) and B <= max(self.portion_graphs) and
+                (rows is None or list(rows) == list(range(B))) and
+                all(s.num_computed // self.block_size + 1 <= self._graph_mb for s, _ in batch)):
+            return self._replay_decode(batch)
         ids, pos, step = self.prepare_portions(batch)
         seq_ops.set_step(step)
         try:

@@ -47,8 +47,11 @@ class RoutedExperts(nn.Module):
         self.w_gu = nn.Parameter(torch.empty(experts, 2 * ff, width), requires_grad=False)
         self.w_down = nn.Parameter(torch.empty(experts, width, ff), requires_grad=False)
         self.shared = shared
+        self._tiled = None         # the expert weights in the layout the matrix-core kernels stream (made at the first step)
 
     def forward(self, h):
+        if self._tiled is None and h.is_cuda and h.dtype == torch.bfloat16:
+            self._tiled = (seq_ops.tile_expert_weights(self.w_gu, 2), seq_ops.tile_expert_weights(self.w_down))
         idx, wts = seq_ops.moe_route(h, self.router, self.top, self.groups, self.keep)
         shared = self.shared(h) if self.shared is not None else None
-        return seq_ops.moe_experts(h, idx, wts, self.w_gu, self.w_down, self.limit, self.alpha, shared)
+        return seq_ops.moe_experts(h, idx, wts, self.w_gu, self.w_down, self.limit, self.alpha, shared, tiled=self._tiled)

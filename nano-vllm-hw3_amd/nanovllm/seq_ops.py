@@ -177,11 +177,25 @@ def moe_route(h, router_w, top, groups=1, keep=1):
 TILES128_MIN_ROWS_PER_EXPERT = 64
 
 
-def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702, shared=None, form=None):
+def tile_expert_weights(w, parts=1):
+    """Expert weights [E, parts * N, K] (K contiguous) -> the layout the matrix-core expert kernels stream: blocks of
+    32 rows x 64 k (4 KB) in the order (expert, part, row block, k step), inside a block chunk s (8 k) of lane L =
+    32 hi + row at 16 (64 s + L) bytes with k = 64 step + 32 hi + 8 s: every load of a wave is one contiguous KB, where
+    the row-major matrix would be touched in 32 pieces a row apart.  Rows and k are zero-padded to whole blocks."""
+    E, PN, K = w.shape
+    N = PN // parts
+    NB, KS = (N + 31) // 32, (K + 63) // 64
+    x = torch.nn.functional.pad(w.view(E, parts, N, K), (0, KS * 64 - K, 0, NB * 32 - N))
+    x = x.view(E, parts, NB, 32, KS, 2, 4, 8).permute(0, 1, 2, 4, 6, 5, 3, 7)      # [E, parts, NB, KS, s, hi, row, 8]
+    return x.contiguous()
+
+
+def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702, shared=None, form=None, tiled=None):
     """y[t] = sum_k wts[t, k] * expert_{idx[t, k]}(h[t]) (+ shared[t]); w_gu [E, 2F, W] (gate rows then up rows),
     w_down [E, W, F]; an expert is a clamped GLU between its two products.  ``form``: "pairs" | "grouped" | "tiles128"
     forces one; by default float32 runs pair by pair and bf16 grouped by expert on the matrix cores, in tiles of 32 rows
-    for small groups (decode) and of 128 rows for large ones (prefill)."""
+    for small groups (decode) and of 128 rows for large ones (prefill).  ``tiled`` = (tile_expert_weights(w_gu, 2),
+    tile_expert_weights(w_down)), what the grouped forms read (made here when the caller does not keep them)."""
     if not h.is_cuda:
         return cpu_ops.moe_experts(h, idx, wts, w_gu, w_down, limit, alpha, shared)
     SM.require_cuda(h, w_gu.dtype, "h")
@@ -203,7 +217,8 @@ def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702, shared=None, form
         prod = torch.empty((rows * n, W), dtype=h.dtype, device=h.device)
         act = torch.empty((rows * n, F), dtype=h.dtype, device=h.device)
         fn = lib.sm_moe_grouped if form == "grouped" else lib.sm_moe_tiles128
-        SM.check(fn(h.data_ptr(), idx.data_ptr(), wts.data_ptr(), w_gu.data_ptr(), w_down.data_ptr(),
+        t_gu, t_down = tiled if tiled is not None else (tile_expert_weights(w_gu, 2), tile_expert_weights(w_down))
+        SM.check(fn(h.data_ptr(), idx.data_ptr(), wts.data_ptr(), t_gu.data_ptr(), t_down.data_ptr(),
                                     SM.ptr(shared), limit, alpha, y.data_ptr(), T, top, E, W, F, row_pair.data_ptr(),
                     tile_expert.data_ptr(), pair_row.data_ptr(), act.data_ptr(), prod.data_ptr(), _dev(h)))
         return y

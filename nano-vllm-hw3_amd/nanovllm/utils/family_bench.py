@@ -61,7 +61,7 @@ def engine_throughput(family, size, prefill_seqs=8, prefill_len=1024, decode_seq
     from nanovllm.engine.sequence import ACTIVE, Sequence
     width, heads, ff, layers, rank = SIZES[size]
     cfg = pasizen_config(width, heads, ff, layers, rank) if family == "pasizen" else qwen3_config(width, heads, ff, layers)
-    llm = LLM(_model_dir(cfg), load_format="dummy", enforce_eager=family == "pasizen", max_model_len=2048,
+    llm = LLM(_model_dir(cfg), load_format="dummy", enforce_eager=False, max_model_len=2048,
               max_num_seqs=decode_seqs, max_num_batched_tokens=prefill_seqs * prefill_len, gpu_memory_utilization=0.5)
     g = torch.Generator().manual_seed(0)
     runner, sch = llm.model_runner, llm.scheduler
@@ -89,7 +89,10 @@ def engine_throughput(family, size, prefill_seqs=8, prefill_len=1024, decode_seq
         for s in dec:
             s.num_computed = decode_ctx
             assert sch.reserve_portion(s, 1)
-        res["decode_s"] = _timed(lambda: runner.run_portions([(s, 1) for s in dec]), reps * 4)
+        res["decode_s"] = _timed(lambda: runner.run_portions([(s, 1) for s in dec]), reps * 4)       # hipGraph replay
+        graphs, runner.portion_graphs = runner.portion_graphs, {}
+        res["decode_eager_s"] = _timed(lambda: runner.run_portions([(s, 1) for s in dec]), reps * 4)
+        runner.portion_graphs = graphs
     else:
         pre = seqs_of(prefill_seqs, prefill_len)
         for s in pre:
@@ -214,15 +217,16 @@ def kernel_table(width=2048, heads=16, rank=256, ff=6144, T=8192, seq=1024, B=64
     w_gu, w_down = r(E, 2 * F, width), r(E, width, F)
     add("sm_moe_route (T=%d, E=%d)" % (T, E), "-", _event_time(lambda: seq_ops.moe_route(h, rw, top, 4, 2)), bytes_=T * width * 2)
     idx, wts = seq_ops.moe_route(h, rw, top, 4, 2)
+    tiled = (seq_ops.tile_expert_weights(w_gu, 2), seq_ops.tile_expert_weights(w_down))
     wgu_d, wd_d = r(2 * ff, width), r(width, ff)
     add("sm_moe_grouped (T=%d, top %d of %d, F=%d)" % (T, top, E, F), "bf16 GEMM of the dense MLP (hipBLASLt)",
-        _event_time(lambda: seq_ops.moe_experts(h, idx, wts, w_gu, w_down, 7.0, form="grouped"), 5), flops=T * top * 6 * width * F)
+        _event_time(lambda: seq_ops.moe_experts(h, idx, wts, w_gu, w_down, 7.0, form="grouped", tiled=tiled), 5), flops=T * top * 6 * width * F)
     add("sm_moe_tiles128 (T=%d, top %d of %d, F=%d)" % (T, top, E, F), "bf16 GEMM of the dense MLP (hipBLASLt)",
-        _event_time(lambda: seq_ops.moe_experts(h, idx, wts, w_gu, w_down, 7.0, form="tiles128"), 5), flops=T * top * 6 * width * F)
+        _event_time(lambda: seq_ops.moe_experts(h, idx, wts, w_gu, w_down, 7.0, form="tiles128", tiled=tiled), 5), flops=T * top * 6 * width * F)
     hm = h[:512].contiguous()
     idx_m, wts_m = seq_ops.moe_route(hm, rw, top, 4, 2)
     add("sm_moe_grouped (T=512)", "bf16 GEMM of the dense MLP (hipBLASLt)",
-        _event_time(lambda: seq_ops.moe_experts(hm, idx_m, wts_m, w_gu, w_down, 7.0, form="grouped"), 5), flops=512 * top * 6 * width * F,
+        _event_time(lambda: seq_ops.moe_experts(hm, idx_m, wts_m, w_gu, w_down, 7.0, form="grouped", tiled=tiled), 5), flops=512 * top * 6 * width * F,
         bytes_=E * 3 * F * width * 2)
     add("dense MLP GEMMs, hipBLASLt (T=512)", "-",
         _event_time(lambda: torch.nn.functional.linear(torch.nn.functional.linear(hm, wgu_d)[:, :ff], wd_d), 5), flops=512 * 6 * width * ff,
@@ -233,7 +237,7 @@ def kernel_table(width=2048, heads=16, rank=256, ff=6144, T=8192, seq=1024, B=64
     idx_d, wts_d = seq_ops.moe_route(hd, rw, top, 4, 2)
     touched = len(torch.unique(idx_d))
     add("sm_moe_grouped (T=%d: decode)" % B, "bf16 GEMM of the dense MLP (hipBLASLt)",
-        _event_time(lambda: seq_ops.moe_experts(hd, idx_d, wts_d, w_gu, w_down, 7.0, form="grouped")), bytes_=touched * 3 * F * width * 2)
+        _event_time(lambda: seq_ops.moe_experts(hd, idx_d, wts_d, w_gu, w_down, 7.0, form="grouped", tiled=tiled)), bytes_=touched * 3 * F * width * 2)
     add("dense MLP GEMMs, hipBLASLt (T=%d: decode)" % B, "-",
         _event_time(lambda: torch.nn.functional.linear(torch.nn.functional.linear(hd, wgu_d)[:, :ff], wd_d)), bytes_=3 * ff * width * 2)
     return rows
