@@ -218,9 +218,9 @@ def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702, shared=None, form
         act = torch.empty((rows * n, F), dtype=h.dtype, device=h.device)
         fn = lib.sm_moe_grouped if form == "grouped" else lib.sm_moe_tiles128
         t_gu, t_down = tiled if tiled is not None else (tile_expert_weights(w_gu, 2), tile_expert_weights(w_down))
-        SM.check(fn(h.data_ptr(), idx.data_ptr(), wts.data_ptr(), t_gu.data_ptr(), t_down.data_ptr(),
-                                    SM.ptr(shared), limit, alpha, y.data_ptr(), T, top, E, W, F, row_pair.data_ptr(),
-                    tile_expert.data_ptr(), pair_row.data_ptr(), act.data_ptr(), prod.data_ptr(), _dev(h)))
+        SM.check(fn(h.data_ptr(), idx.data_ptr(), wts.data_ptr(), t_gu.data_ptr(), t_down.data_ptr(), SM.ptr(shared), limit, alpha,
+                    y.data_ptr(), T, top, E, W, F, row_pair.data_ptr(), tile_expert.data_ptr(), pair_row.data_ptr(),
+                    act.data_ptr(), prod.data_ptr(), _dev(h)))
         return y
     assert form == "pairs", form
     act = torch.empty((T * top, F), dtype=h.dtype, device=h.device)

@@ -16,9 +16,9 @@ import torch
 
 
 def replay(model, dtype, out_dir, max_tokens, lines, device="cuda", max_live=4, log=sys.stdout):
+    from nanovllm.config import Config
     from nanovllm.engine.llm_engine import LLMEngine
     from nanovllm.engine.sequence import ACTIVE, Sequence
-    from nanovllm.config import Config
     cfg0 = Config(model, device=device, dtype=dtype, enforce_eager=True)
     if not cfg0.runs_portions:
         raise SystemExit("trace replay needs a model family that is stepped with portions of sequences")
