@@ -1,0 +1,108 @@
+/*
+ * libhymix - MI355X (gfx950) kernels of a decoder that mixes rotary attention layers with delta-rule recurrent
+ * layers on a float32 residual: scaled embedding, the gated sublayer boundary with RMS norms on both sides,
+ * token shift with a carried row per sequence, the preparation of q/k/v (projection norms, partial rotation,
+ * unit-norm heads, value blending between layers, paged cache store), attention over the paged cache with
+ * sinks and sliding windows that keep the first tokens, the generalized delta rule with a float32 state per
+ * sequence, and squared ReLU.
+ *
+ * Conventions (those of libqlinear and libseqmix): all pointers are DEVICE pointers owned by the caller,
+ * matrices are row-major and dense unless a stride (in elements) is named; `stream` is a hipStream_t passed as
+ * void*; nothing here allocates, frees or synchronises, so every call may be captured into a hipGraph;
+ * 0 = launched, a negative HM_E* code = rejected before any launch, with a message from hm_last_error().
+ *
+ * `dtype` selects the storage type of activations, weights and caches: HM_F32 or HM_BF16.  Whatever the storage
+ * type, the residual, norms, gates, angles, attention scores and weights, and everything inside the recurrence
+ * are float32.
+ *
+ * A step's batch: B sequences contribute portions of consecutive tokens, T tokens in all, packed sequence after
+ * sequence.  tok_seq[t] = index of the token's sequence in the step, tok_pos[t] = its position in the sequence,
+ * qstart[b] = first row of sequence b (qstart[B] = T), seq_pos0[b] = position of its first token in this step,
+ * seq_slot[b] = its state slot, slot_mapping[t] = cache row (block * block_size + offset) of the token,
+ * block_tables [B, max_blocks].
+ */
+#ifndef HYMIX_H
+#define HYMIX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HM_F32 0
+#define HM_BF16 1
+
+#define HM_OK 0
+#define HM_EINVAL (-1)
+#define HM_ESHAPE (-2)
+#define HM_EWORKSPACE (-3)
+#define HM_ELAUNCH (-4)
+
+int hm_version(void);
+const char* hm_last_error(void);
+
+/* x[t] = embed[ids[t]] * scale (f32). */
+int hm_embed_scaled(int dtype, const int64_t* ids, const void* embed, float scale, float* x, int64_t T, int W, void* stream);
+
+/* The boundary between two sublayers, per token t, in one launch (x is [T, W] f32, updated in place):
+ *   y != NULL:       z = y[t] * sigmoid(gate[t] + gate_bias);  x[t] += mult * z / sqrt(mean(z^2) + eps) * post_w
+ *   next_w != NULL:  h_out[t] = x[t] / sqrt(mean(x[t]^2) + eps) * next_w
+ *   carry_src != NULL: for the last token of every sequence's portion, carry_state[seq_slot * slot_stride + :] = carry_src[t]
+ * gate rows are gate_stride elements apart. */
+int hm_sublayer_close(int dtype, float* x, const void* y, const void* gate, int64_t gate_stride, const void* gate_bias,
+                      const void* post_w, float mult, const void* next_w, float eps, void* h_out, const void* carry_src,
+                      void* carry_state, int64_t slot_stride, const int32_t* tok_seq, const int32_t* qstart,
+                      const int32_t* seq_slot, int64_t T, int W, void* stream);
+
+/* out[t] = h[t] + (prev - h[t]) * mu;  prev = h[t-1] inside a portion, state[seq_slot * slot_stride + :] at a portion's
+ * start, zero at position 0. */
+int hm_token_shift(int dtype, const void* h, const void* mu, const void* state, int64_t slot_stride, const int32_t* tok_seq,
+                   const int32_t* tok_pos, const int32_t* qstart, const int32_t* seq_slot, void* out, int64_t T, int W,
+                   void* stream);
+
+/* out[t, c] = max(z[t, c], 0)^2; z rows are z_stride elements apart. */
+int hm_relu_squared(int dtype, const void* z, int64_t z_stride, void* out, int64_t T, int F, void* stream);
+
+/* qkv [T, H*D + G*D + G*V] (rows row_stride apart), per token:
+ *   q_norm_w / k_norm_w != NULL: RMS norm over the whole q (k) projection with that weight;
+ *   the first 2 * rot_half channels of every q and k head turn by tok_pos * inv_freq[i] (channel i with i + rot_half);
+ *   unit_norm: every rotated head divided by its RMS;
+ *   v_first != NULL: v <- (1 - lam[0]) v + lam[0] v_first[t];
+ *   k and v go to row slot_mapping[t] of the caches [rows, G, D] / [rows, G, V] (a negative row: not stored);
+ *   q_out [T, H, D]. */
+int hm_qkv_prepare(int dtype, const void* qkv, int64_t row_stride, int H, int G, int D, int V, const void* q_norm_w,
+                   const void* k_norm_w, float eps, const float* inv_freq, int rot_half, int unit_norm, const int32_t* tok_pos,
+                   const int32_t* slot_mapping, void* k_cache, void* v_cache, const void* v_first, int64_t v_first_stride,
+                   const float* lam, void* q_out, int64_t T, void* stream);
+
+/* Attention of q [T, H, D] over the paged caches, any sizes, f32 arithmetic: the token at position i sees key j <= i,
+ * and with window > 0 only if i - j < window or j < keep_first.  sink != NULL (f32 [H]): exp(sink[h]) joins the softmax
+ * denominator.  o [T, H, V]. */
+int hm_attn_rows(int dtype, const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables,
+                 const int32_t* tok_seq, const int32_t* tok_pos, const float* sink, int window, int keep_first, float scale,
+                 void* o, int64_t T, int H, int G, int D, int V, int block_size, int max_blocks, void* stream);
+
+/* prep [T, H, 5, D] f32 = decay | a*u | u | k | r from the columns r_off, k_off, a_off (H*D wide) and z_off (rank wide) of
+ * proj:  decay = exp(-decay_scale * sigmoid(w2 tanh(z) + w0)), a = sigmoid(a_pre + a_bias), u = k / sqrt(sum k^2 + unit_eps)
+ * per head.  w2 [H*D, rank]. */
+int hm_delta_prepare(int dtype, const void* proj, int64_t row_stride, int r_off, int k_off, int a_off, int z_off,
+                     const void* w2, const void* w0, const void* a_bias, int rank, float decay_scale, float unit_eps,
+                     float* prep, int64_t T, int H, int D, void* stream);
+
+/* For every sequence b and head, over the tokens of its portion in order:
+ *   S <- diag(decay) S - (a u)(u^T S) + k v^T (both terms from the old S);  o[t] = S^T r
+ * state f32 [slots, H, D, D] is read at the start unless seq_pos0[b] == 0 (then S = 0) and written at the end.
+ * v [T, H*D] in the storage type, rows v_stride apart.  o f32 [T, H, D].  D <= 256. */
+int hm_delta_recurrence(int dtype, const float* prep, const void* v, int64_t v_stride, float* state, const int32_t* qstart,
+                        const int32_t* seq_pos0, const int32_t* seq_slot, float* o, int B, int H, int D, void* stream);
+
+/* out[t, h*D + i] = o[t, h, i] / sqrt(mean_i o[t, h]^2 + eps) * norm_w[h*D + i] * sigmoid(g[t, h*D + i]). */
+int hm_delta_gate_norm(int dtype, const float* o, const void* g, int64_t g_stride, const void* norm_w, float eps, void* out,
+                       int64_t T, int H, int D, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

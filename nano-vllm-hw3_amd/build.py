@@ -1,10 +1,12 @@
 """Build the package's HIP libraries (gfx950) in-tree with hipcc.  No GPU is needed to build.
 
-Two libraries, each from its own folder of translation units, so that a model only waits for what it runs on:
+Three libraries, each from its own folder of translation units, so that a model only waits for what it runs on:
   qlinear  csrc/*.hip         -> nanovllm/_lib/libqlinear.so   (quantized linears, Qwen3 operators, attention)
   seqmix   csrc/seqmix/*.hip  -> nanovllm/_lib/libseqmix.so    (multi-stream residuals, short convolutions, latent
                                                                 attention, PolyNorm / clamped GLU, expert routing)
-``python build.py [--force] [qlinear|seqmix]`` builds one of them, or both without a name."""
+  hymix    csrc/hymix/*.hip   -> nanovllm/_lib/libhymix.so     (gated residual, token shift, rotary attention with sinks
+                                                                and windows over a paged cache, delta-rule recurrence)
+``python build.py [--force] [qlinear|seqmix|hymix]`` builds one of them, or all without a name."""
 import os
 import shutil
 import subprocess
@@ -16,12 +18,14 @@ CSRC = os.path.join(HERE, "csrc")
 OUT_DIR = os.path.join(HERE, "nanovllm", "_lib")
 LIB = os.path.join(OUT_DIR, "libqlinear.so")
 SEQMIX_LIB = os.path.join(OUT_DIR, "libseqmix.so")
+HYMIX_LIB = os.path.join(OUT_DIR, "libhymix.so")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-fno-gpu-rdc"]
 # the packed-f32 VALU forms stay off in the newer library (plain f32 code only)
 NO_PACKED_F32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 TARGETS = {
     "qlinear": dict(src=CSRC, lib=LIB, header="qlinear.h", flags=FLAGS, obj=""),
     "seqmix": dict(src=os.path.join(CSRC, "seqmix"), lib=SEQMIX_LIB, header="seqmix.h", flags=FLAGS + NO_PACKED_F32, obj="seqmix_"),
+    "hymix": dict(src=os.path.join(CSRC, "hymix"), lib=HYMIX_LIB, header="hymix.h", flags=FLAGS + NO_PACKED_F32, obj="hymix_"),
 }
 
 
@@ -40,7 +44,7 @@ def _stale(target, deps):
 
 
 def build(force=False, verbose=True, target="qlinear"):
-    """Compile one library (``target`` = "qlinear" | "seqmix") or both ("all"); returns the path of the (last) library."""
+    """Compile one library (``target`` = "qlinear" | "seqmix") or all of them ("all"); returns the path of the (last) library."""
     if target == "all":
         for name in TARGETS:
             lib = build(force, verbose, name)

@@ -1,0 +1,201 @@
+// Rotary attention over a paged key/value cache.  This file holds the per-token preparation launch (norms of q and k,
+// rotation, value blending, cache store) and the portable attention kernel (any head sizes, f32 or bf16 storage, f32
+// arithmetic) with the masks and sinks the layers can ask for; the matrix-core kernels are in hm_attn_mfma.hip.
+#include "hm_common.h"
+
+namespace hm {
+
+// One workgroup per token.  q and k travel through LDS as f32: [H*D] then [G*D].
+template <typename T>
+__global__ __launch_bounds__(256) void qkv_prepare_kernel(const T* __restrict__ qkv, int64_t row_stride, int H, int G, int D,
+                                                          int V, const T* __restrict__ q_norm_w, const T* __restrict__ k_norm_w,
+                                                          float eps, const float* __restrict__ inv_freq, int rot_half,
+                                                          int unit_norm, const int32_t* __restrict__ tok_pos,
+                                                          const int32_t* __restrict__ slot_mapping, T* __restrict__ k_cache,
+                                                          T* __restrict__ v_cache, const T* __restrict__ v_first,
+                                                          int64_t v_first_stride, const float* __restrict__ lam,
+                                                          T* __restrict__ q_out) {
+    extern __shared__ float qk[];
+    __shared__ float red[16];
+    const int64_t t = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int nq = H * D, nk = G * D, nv = G * V;
+    const T* row = qkv + (size_t)t * row_stride;
+    float sq = 0.f, sk = 0.f;
+    for (int c = tid; c < nq + nk; c += 256) {
+        const float v = to_f(row[c]);
+        qk[c] = v;
+        if (c < nq) sq += v * v; else sk += v * v;
+    }
+    if (q_norm_w != nullptr) {                 // RMS norm over the whole projection, with a weight
+        sq = block_sum(sq, red);
+        sk = block_sum(sk, red);
+        const float rq = 1.f / sqrtf(sq / (float)nq + eps), rk = 1.f / sqrtf(sk / (float)nk + eps);
+        for (int c = tid; c < nq + nk; c += 256)
+            qk[c] = c < nq ? qk[c] * rq * to_f(q_norm_w[c]) : qk[c] * rk * to_f(k_norm_w[c - nq]);
+    }
+    __syncthreads();
+    const float pos = (float)tok_pos[t];
+    for (int e = tid; e < (H + G) * rot_half; e += 256) {       // one thread per rotated pair
+        const int hh = e / rot_half, i = e - hh * rot_half;
+        float s, c;
+        sincosf(pos * inv_freq[i], &s, &c);
+        float* p = qk + (size_t)hh * D;
+        const float a = p[i], b = p[i + rot_half];
+        p[i] = a * c - b * s;
+        p[i + rot_half] = b * c + a * s;
+    }
+    __syncthreads();
+    if (unit_norm) {                           // every head divided by its RMS; one wave per head
+        for (int hh = wave; hh < H + G; hh += 4) {
+            float* p = qk + (size_t)hh * D;
+            float ss = 0.f;
+            for (int i = lane; i < D; i += 64) ss += p[i] * p[i];
+            ss = wave_sum(ss);
+            const float r = 1.f / sqrtf(ss / (float)D + eps);
+            for (int i = lane; i < D; i += 64) p[i] *= r;
+        }
+        __syncthreads();
+    }
+    for (int c = tid; c < nq; c += 256) q_out[(size_t)t * nq + c] = from_f<T>(qk[c]);
+    const int slot = slot_mapping[t];
+    if (slot < 0) return;
+    for (int c = tid; c < nk; c += 256) k_cache[(size_t)slot * nk + c] = from_f<T>(qk[nq + c]);
+    const T* vr = row + nq + nk;
+    if (v_first != nullptr) {
+        const float l = lam[0];
+        const T* fr = v_first + (size_t)t * v_first_stride;
+        for (int c = tid; c < nv; c += 256)
+            v_cache[(size_t)slot * nv + c] = from_f<T>((1.f - l) * to_f(vr[c]) + l * to_f(fr[c]));
+    } else {
+        for (int c = tid; c < nv; c += 256) v_cache[(size_t)slot * nv + c] = vr[c];
+    }
+}
+
+constexpr int kRowChunk = 64;      // keys per step of the portable kernel
+
+// One workgroup per (token, head).  The keys a query at position i sees are enumerated as one list: with a window, the
+// kept first tokens that lie before the window, then the window; without, all of 0..i.  The order of the sums depends on
+// the position alone.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_rows_kernel(const T* __restrict__ q, const T* __restrict__ k_cache,
+                                                        const T* __restrict__ v_cache, const int32_t* __restrict__ block_tables,
+                                                        const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
+                                                        const float* __restrict__ sink, int window, int keep_first, float scale,
+                                                        T* __restrict__ o, int H, int G, int D, int V, int block_size,
+                                                        int max_blocks) {
+    extern __shared__ float q_lds[];                 // D floats
+    __shared__ float s_lds[kRowChunk];
+    __shared__ int row_lds[kRowChunk];
+    const int64_t t = blockIdx.x;
+    const int hd = blockIdx.y, g = hd / (H / G);
+    const int b = tok_seq[t], n = tok_pos[t] + 1;    // keys 0 .. n-1 are causal
+    const int lo = window > 0 ? max(0, n - window) : 0;
+    const int kept = window > 0 ? min(keep_first, lo) : 0;
+    const int total = kept + (n - lo);
+    const int32_t* table = block_tables + (size_t)b * max_blocks;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const T* qr = q + ((size_t)t * H + hd) * D;
+    for (int c = tid; c < D; c += 256) q_lds[c] = to_f(qr[c]);
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};             // channels tid, tid + 256, ... of the output row
+    float m_run = -INFINITY, l_run = 0.f;
+    for (int k0 = 0; k0 < total; k0 += kRowChunk) {
+        __syncthreads();                             // q_lds ready / previous chunk's s_lds and row_lds consumed
+        if (tid < kRowChunk) {
+            const int e = k0 + tid;
+            const int key = e < kept ? e : lo + (e - kept);
+            row_lds[tid] = e < total ? table[key / block_size] * block_size + key % block_size : -1;
+        }
+        __syncthreads();
+        for (int kk = wave; kk < kRowChunk; kk += 4) {
+            const int row = row_lds[kk];
+            float d = 0.f;
+            if (row >= 0) {
+                const T* kr = k_cache + ((size_t)row * G + g) * D;
+                for (int c = lane; c < D; c += 64) d += q_lds[c] * to_f(kr[c]);
+            }
+            d = wave_sum(d);
+            if (lane == 0) s_lds[kk] = row >= 0 ? d * scale : -INFINITY;
+        }
+        __syncthreads();
+        float mx = m_run;
+        for (int kk = 0; kk < kRowChunk; ++kk) mx = fmaxf(mx, s_lds[kk]);
+        const float alpha = expf(m_run - mx);        // first chunk: exp(-inf) = 0
+        float psum = 0.f;
+        for (int r = 0; r < 4; ++r) acc[r] *= alpha;
+        for (int kk = 0; kk < kRowChunk; ++kk) {
+            const int row = row_lds[kk];
+            if (row < 0) break;
+            const float p = expf(s_lds[kk] - mx);
+            psum += p;
+            const T* vr = v_cache + ((size_t)row * G + g) * V;
+            for (int r = 0; r < 4; ++r) {
+                const int c = tid + 256 * r;
+                if (c < V) acc[r] += p * to_f(vr[c]);
+            }
+        }
+        l_run = l_run * alpha + psum;
+        m_run = mx;
+    }
+    float inv;
+    if (sink != nullptr) {                           // one more term in the denominator, no value
+        const float sk = sink[hd], mx = fmaxf(m_run, sk), alpha = expf(m_run - mx);
+        for (int r = 0; r < 4; ++r) acc[r] *= alpha;
+        inv = 1.f / (l_run * alpha + expf(sk - mx));
+    } else {
+        inv = 1.f / l_run;
+    }
+    T* orow = o + ((size_t)t * H + hd) * V;
+    for (int r = 0; r < 4; ++r) {
+        const int c = tid + 256 * r;
+        if (c < V) orow[c] = from_f<T>(acc[r] * inv);
+    }
+}
+
+}  // namespace hm
+
+using namespace hm;
+
+extern "C" int hm_qkv_prepare(int dtype, const void* qkv, int64_t row_stride, int H, int G, int D, int V, const void* q_norm_w,
+                              const void* k_norm_w, float eps, const float* inv_freq, int rot_half, int unit_norm,
+                              const int32_t* tok_pos, const int32_t* slot_mapping, void* k_cache, void* v_cache,
+                              const void* v_first, int64_t v_first_stride, const float* lam, void* q_out, int64_t T,
+                              void* stream) {
+    if (T < 0 || H < 1 || G < 1 || D < 1 || V < 1 || H % G != 0 || rot_half < 0 || 2 * rot_half > D ||
+        row_stride < (int64_t)(H + G) * D + (int64_t)G * V || (!q_norm_w) != (!k_norm_w) || (rot_half > 0 && !inv_freq) ||
+        (v_first && (!lam || v_first_stride < (int64_t)G * V)) ||
+        (T > 0 && (!qkv || !tok_pos || !slot_mapping || !k_cache || !v_cache || !q_out))) {
+        set_error("hm_qkv_prepare: bad argument");
+        return HM_EINVAL;
+    }
+    const size_t lds = (size_t)(H + G) * D * 4;
+    if (lds > 60 * 1024) { set_error("hm_qkv_prepare: (heads + kv_heads) * dim = %d does not fit the row buffer", (H + G) * D); return HM_ESHAPE; }
+    if (T == 0) return HM_OK;
+    HM_DISPATCH(dtype, "hm_qkv_prepare",
+                hipLaunchKernelGGL(qkv_prepare_kernel<DT>, dim3((unsigned)T), dim3(256), lds, as_stream(stream), (const DT*)qkv,
+                                   row_stride, H, G, D, V, (const DT*)q_norm_w, (const DT*)k_norm_w, eps, inv_freq, rot_half,
+                                   unit_norm, tok_pos, slot_mapping, (DT*)k_cache, (DT*)v_cache, (const DT*)v_first,
+                                   v_first_stride, lam, (DT*)q_out));
+    HM_CHECK_LAUNCH("hm_qkv_prepare");
+    return HM_OK;
+}
+
+extern "C" int hm_attn_rows(int dtype, const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables,
+                            const int32_t* tok_seq, const int32_t* tok_pos, const float* sink, int window, int keep_first,
+                            float scale, void* o, int64_t T, int H, int G, int D, int V, int block_size, int max_blocks,
+                            void* stream) {
+    if (T < 0 || H < 1 || G < 1 || H % G != 0 || D < 1 || V < 1 || block_size < 1 || max_blocks < 1 || window < 0 || keep_first < 0 ||
+        (T > 0 && (!q || !k_cache || !v_cache || !block_tables || !tok_seq || !tok_pos || !o))) {
+        set_error("hm_attn_rows: bad argument");
+        return HM_EINVAL;
+    }
+    if (V > 1024 || D > 8192 || H > 65535) { set_error("hm_attn_rows: vdim <= 1024, dim <= 8192 and heads <= 65535"); return HM_ESHAPE; }
+    if (T == 0) return HM_OK;
+    dim3 grid((unsigned)T, (unsigned)H);
+    HM_DISPATCH(dtype, "hm_attn_rows",
+                hipLaunchKernelGGL(attn_rows_kernel<DT>, grid, dim3(256), (size_t)D * 4, as_stream(stream), (const DT*)q,
+                                   (const DT*)k_cache, (const DT*)v_cache, block_tables, tok_seq, tok_pos, sink, window,
+                                   keep_first, scale, (DT*)o, H, G, D, V, block_size, max_blocks));
+    HM_CHECK_LAUNCH("hm_attn_rows");
+    return HM_OK;
+}

@@ -189,3 +189,129 @@ def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha, shared):
     if shared is not None:
         y = y + shared.float()
     return y.to(h.dtype)
+
+
+# ---- plumbing counterparts of nanovllm/hy_ops.py --------------------------------------------------------------------
+def _unit_rms(x, eps):
+    return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+
+
+def embed_scaled(ids, embed, scale):
+    return embed[ids].float() * scale
+
+
+def sublayer_close(x, y, gate, gate_bias, post_w, mult, next_w, eps, dtype, carry):
+    if y is not None:
+        z = y.float() * torch.sigmoid(gate.float() + gate_bias.float())
+        x.add_(mult * _unit_rms(z, eps) * post_w.float())
+    if carry is not None:
+        src, state, layer, ctx = carry
+        last = (ctx.qstart[1:] - 1).long()
+        state[ctx.seq_slot.long(), layer] = src[last].to(state.dtype)
+    if next_w is None:
+        return None
+    return (_unit_rms(x, eps) * next_w.float()).to(dtype)
+
+
+def token_shift(h, mu, state, layer, ctx):
+    hf = h.float()
+    prev = torch.cat([torch.zeros_like(hf[:1]), hf[:-1]], 0)
+    first = ctx.qstart[:-1].long()
+    carried = state[ctx.seq_slot.long(), layer].float()
+    carried = carried * (ctx.seq_pos0 > 0).float()[:, None]
+    prev[first] = carried
+    return (hf + (prev - hf) * mu.float()).to(h.dtype)
+
+
+def rotate_half_partial(x, pos, inv_freq):
+    """x f32 [T, heads, D]: the first 2 * len(inv_freq) channels of every head turn by pos * inv_freq."""
+    half = inv_freq.numel()
+    ang = pos.float()[:, None] * inv_freq[None, :]
+    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    a, b = x[..., :half], x[..., half:2 * half]
+    return torch.cat([a * c - b * s, b * c + a * s, x[..., 2 * half:]], -1)
+
+
+def qkv_prepare(qkv, H, G, D, V, q_norm_w, k_norm_w, eps, inv_freq, unit_norm, ctx, k_cache, v_cache, v_first, lam):
+    T = qkv.shape[0]
+    q, k, v = qkv.float().split([H * D, G * D, G * V], -1)
+    if q_norm_w is not None:
+        q, k = _unit_rms(q, eps) * q_norm_w.float(), _unit_rms(k, eps) * k_norm_w.float()
+    q, k = q.reshape(T, H, D), k.reshape(T, G, D)
+    q, k = rotate_half_partial(q, ctx.tok_pos, inv_freq), rotate_half_partial(k, ctx.tok_pos, inv_freq)
+    if unit_norm:
+        q, k = _unit_rms(q, eps), _unit_rms(k, eps)
+    if v_first is not None:
+        v = (1 - lam.float()) * v + lam.float() * v_first.float()
+    rows = ctx.slot_mapping.long()
+    k_cache.view(-1, G, D)[rows] = k.to(k_cache.dtype)
+    v_cache.view(-1, G, V)[rows] = v.reshape(T, G, V).to(v_cache.dtype)
+    return q.to(qkv.dtype).contiguous()
+
+
+def paged_attention(q, k_cache, v_cache, ctx, scale, sink, window, keep_first):
+    T, H, D = q.shape
+    bs, G, V = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    o = torch.empty((T, H * V), dtype=q.dtype)
+    kr, vr = k_cache.view(-1, G, D), v_cache.view(-1, G, V)
+    qs = ctx.qstart.tolist()
+    for b in range(ctx.num_seqs):
+        a, e = qs[b], qs[b + 1]
+        if e <= a:
+            continue
+        n = int(ctx.ctx_lens[b])
+        j = torch.arange(n)
+        rows = ctx.block_tables[b, j // bs].long() * bs + j % bs
+        kk = kr[rows].float().repeat_interleave(H // G, 1)                       # [n, H, D]
+        vv = vr[rows].float().repeat_interleave(H // G, 1)
+        s = torch.einsum("thd,nhd->thn", q[a:e].float(), kk) * scale
+        i = ctx.tok_pos[a:e].long()[:, None]
+        ok = j[None, :] <= i
+        if window > 0:
+            ok &= ((i - j[None, :]) < window) | (j[None, :] < keep_first)
+        s = s.masked_fill(~ok[:, None, :], float("-inf"))
+        if sink is not None:
+            s = torch.cat([s, sink.float()[None, :, None].expand(e - a, H, 1)], -1)
+        p = torch.softmax(s, -1)[..., :n]
+        o[a:e] = torch.einsum("thn,nhv->thv", p, vv).reshape(e - a, H * V).to(q.dtype)
+    return o
+
+
+def delta_prepare(proj, cols, w2, w0, a_bias, H, D, decay_scale):
+    T = proj.shape[0]
+    pf = proj.float()
+    r, k, a_pre, z = (pf[:, c:c + n] for c, n in cols)
+    decay = torch.exp(-decay_scale * torch.sigmoid(torch.tanh(z) @ w2.float().t() + w0.float()))
+    a = torch.sigmoid(a_pre + a_bias.float())
+    kh = k.reshape(T, H, D)
+    u = kh / torch.sqrt(kh.pow(2).sum(-1, keepdim=True) + 1e-6)
+    return torch.stack([decay.reshape(T, H, D), a.reshape(T, H, D) * u, u, kh, r.reshape(T, H, D)], 2).contiguous()
+
+
+def delta_recurrence(prep, v, state, ctx):
+    T, H, _, D = prep.shape
+    o = torch.empty((T, H, D), dtype=torch.float32)
+    vf = v.float().reshape(T, H, D)
+    qs = ctx.qstart.tolist()
+    for b in range(ctx.num_seqs):
+        a, e = qs[b], qs[b + 1]
+        if e <= a:
+            continue
+        slot = int(ctx.seq_slot[b])
+        S = state[slot].clone() if int(ctx.seq_pos0[b]) > 0 else torch.zeros_like(state[slot])
+        for t in range(a, e):
+            decay, au, u, k, r = prep[t].unbind(1)
+            uS = torch.einsum("hi,hij->hj", u, S)
+            S = decay[:, :, None] * S - au[:, :, None] * uS[:, None, :] + k[:, :, None] * vf[t][:, None, :]
+            o[t] = torch.einsum("hij,hi->hj", S, r)
+        state[slot] = S
+    return o
+
+
+def delta_gate_norm(o, g, norm_w, eps, dtype):
+    T, H, D = o.shape
+    return (_unit_rms(o, eps).reshape(T, H * D) * norm_w.float() * torch.sigmoid(g.float())).to(dtype)
+
+
+def relu_squared(z):
+    return torch.relu(z.float()).pow(2).to(z.dtype)

@@ -80,9 +80,11 @@ class ModelRunner:
         runner loads it, sizes the block pool and the state slots, and hands every step a StepContext."""
         cfg, hf = self.config, self.config.hf_config
         if self.on_gpu:
-            from nanovllm import _seqmix
-            _seqmix.build_if_missing()           # a fresh checkout compiles this library (and only it) here
-            _seqmix.load()
+            # a fresh checkout compiles the library this family runs on (and only it) here
+            import importlib
+            native = importlib.import_module("nanovllm._" + getattr(model_cls, "native_library", "seqmix"))
+            native.build_if_missing()
+            native.load()
             # float32 means float32: no reduced-precision matrix mode
             torch.backends.cuda.matmul.allow_tf32 = False
         self.model = model_cls(hf)
@@ -119,7 +121,7 @@ class ModelRunner:
         return offs
 
     def _capture_portion_graphs(self):
-        from nanovllm import _seqmix, seq_ops
+        from nanovllm import seq_ops
         cfg, bs = self.config, self.block_size
         mb = (cfg.max_model_len + bs - 1) // bs
         self._graph_mb = mb
@@ -162,7 +164,8 @@ class ModelRunner:
                 pool = g.pool()
             self.portion_graphs[gb] = dict(graph=g, host=host, pad=pad, dev=dev, offs=offs, logits=logits)
         torch.cuda.synchronize()
-        _seqmix.decode_workspace.pin(self.device)                # the graphs address it: never freed
+        for ws in self.model.workspaces():                       # the graphs address them: never freed
+            ws.pin(self.device)
 
     def _replay_decode(self, batch):
         """A step of single tokens through the captured graph of the smallest bucket that holds it; float32 logits [B, vocab]."""

@@ -1,0 +1,192 @@
+"""Operators of libhymix behind torch tensors: what sits between the matrix products of a decoder that mixes rotary
+attention layers (sinks, sliding windows with kept first tokens, value mixing between layers) with delta-rule recurrent
+layers, on a float32 residual whose sublayers are normalised on both sides, gated, and read a token-shifted input.
+One kernel launch each on the current stream; the step's batch is a nanovllm.seq_ops.StepContext.  CPU tensors go to
+plain-torch counterparts (nanovllm/cpu_ops.py): engine plumbing on a host without a GPU, never a fallback for a GPU tensor."""
+import torch
+
+from nanovllm import _hymix as HM
+from nanovllm import cpu_ops
+from nanovllm.seq_ops import StepContext
+
+
+def _dev(t):
+    return HM.stream_ptr(t.device)
+
+
+def _rows(t, name):
+    """A matrix whose rows may be a column slice of a wider product: unit stride inside a row."""
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise HM.QLinearError(f"{name} must be a matrix with contiguous rows")
+    return t
+
+
+def embed_scaled(ids, embed, scale):
+    """x f32 [T, W] = embed[id] * scale."""
+    if not embed.is_cuda:
+        return cpu_ops.embed_scaled(ids, embed, scale)
+    T, W = ids.numel(), embed.shape[1]
+    x = torch.empty((T, W), dtype=torch.float32, device=embed.device)
+    HM.check(HM.load().hm_embed_scaled(HM.dtype_code(embed.dtype), ids.data_ptr(), embed.data_ptr(), float(scale), x.data_ptr(),
+                                       T, W, _dev(embed)))
+    return x
+
+
+def sublayer_close(x, y, gate, gate_bias, post_w, mult, next_w, eps, dtype, carry=None):
+    """The boundary between two sublayers on a float32 residual x [T, W], per token in one launch:
+      y given:      x <- x + mult * rms_norm(y * sigmoid(gate + gate_bias)) * post_w      (gate: pre-activation, rows may
+                    be a column slice of a wider product)
+      next_w given: returns rms_norm(x) * next_w in ``dtype`` (the next sublayer's input)
+      carry = (src [T, W], state [slots, layers, W], layer, ctx): state[slot of the sequence, layer] <- src[last token of
+                    the sequence's portion] (what a token shift of that layer reads at the next step)."""
+    if not x.is_cuda:
+        return cpu_ops.sublayer_close(x, y, gate, gate_bias, post_w, mult, next_w, eps, dtype, carry)
+    T, W = x.shape
+    h = torch.empty((T, W), dtype=dtype, device=x.device) if next_w is not None else None
+    if y is not None:
+        HM.require_cuda(y, dtype, "y")
+        _rows(gate, "gate")
+    src = state = None
+    tok_seq = qstart = seq_slot = None
+    slot_stride = 0
+    if carry is not None:
+        src, st, layer, ctx = carry
+        HM.require_cuda(src, dtype, "carry source")
+        assert st.dtype == dtype and st.is_contiguous() and st.shape[2] == W
+        state, slot_stride = st[:, layer], st.stride(0)
+        tok_seq, qstart, seq_slot = ctx.tok_seq, ctx.qstart, ctx.seq_slot
+    HM.check(HM.load().hm_sublayer_close(HM.dtype_code(dtype), x.data_ptr(), HM.ptr(y), HM.ptr(gate),
+                                         gate.stride(0) if gate is not None else 0, HM.ptr(gate_bias), HM.ptr(post_w), float(mult),
+                                         HM.ptr(next_w), float(eps), HM.ptr(h), HM.ptr(src), HM.ptr(state), slot_stride,
+                                         HM.ptr(tok_seq), HM.ptr(qstart), HM.ptr(seq_slot), T, W, _dev(x)))
+    return h
+
+
+def token_shift(h, mu, state, layer, ctx: StepContext):
+    """h [T, W] -> h + (h_prev - h) * mu, h_prev = the previous token's h: the row above inside a portion, the sequence's
+    carried row state[slot, layer] at a portion's start, zero at position 0 (a slot is never cleared)."""
+    if not h.is_cuda:
+        return cpu_ops.token_shift(h, mu, state, layer, ctx)
+    HM.require_cuda(h, mu.dtype, "h")
+    T, W = h.shape
+    out = torch.empty_like(h)
+    st = state[:, layer]
+    HM.check(HM.load().hm_token_shift(HM.dtype_code(h.dtype), h.data_ptr(), mu.data_ptr(), st.data_ptr(), state.stride(0),
+                                      ctx.tok_seq.data_ptr(), ctx.tok_pos.data_ptr(), ctx.qstart.data_ptr(),
+                                      ctx.seq_slot.data_ptr(), out.data_ptr(), T, W, _dev(h)))
+    return out
+
+
+def rotary_inv_freq(dims, base, device):
+    """f_i = base^(-2i/dims), i < dims/2, evaluated in float64 and kept in float32."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    return (float(base) ** (-2.0 * i / dims)).to(torch.float32).to(device)
+
+
+def qkv_prepare(qkv, H, G, D, V, q_norm_w, k_norm_w, eps, inv_freq, unit_norm, ctx: StepContext, k_cache, v_cache,
+                v_first=None, lam=None):
+    """From the merged product qkv [T, H*D + G*D + G*V] of a step's tokens, in one launch per token:
+      q_norm_w / k_norm_w given: RMS norm over the WHOLE q (k) projection with that weight;
+      rotation of the first 2 * len(inv_freq) channels of every q and k head by position * inv_freq (channel i paired
+      with channel i + len(inv_freq)), angles in float32;
+      unit_norm: every rotated head of q and k divided by its RMS;
+      v_first given: v <- (1 - lam) v + lam v_first (lam: float32 scalar on the device);
+      k and v are stored at the tokens' cache rows; returns q [T, H, D]."""
+    if not qkv.is_cuda:
+        return cpu_ops.qkv_prepare(qkv, H, G, D, V, q_norm_w, k_norm_w, eps, inv_freq, unit_norm, ctx, k_cache, v_cache,
+                                   v_first, lam)
+    _rows(qkv, "qkv")
+    T = qkv.shape[0]
+    assert qkv.shape[1] == H * D + G * D + G * V and k_cache.dtype == v_cache.dtype == qkv.dtype
+    assert k_cache.shape[2:] == (G, D) and v_cache.shape[2:] == (G, V) and inv_freq.dtype == torch.float32
+    if v_first is not None:
+        _rows(v_first, "v_first")
+        assert v_first.shape == (T, G * V) and lam.dtype == torch.float32
+    q = torch.empty((T, H, D), dtype=qkv.dtype, device=qkv.device)
+    HM.check(HM.load().hm_qkv_prepare(HM.dtype_code(qkv.dtype), qkv.data_ptr(), qkv.stride(0), H, G, D, V, HM.ptr(q_norm_w),
+                                      HM.ptr(k_norm_w), float(eps), inv_freq.data_ptr(), inv_freq.numel(), int(bool(unit_norm)),
+                                      ctx.tok_pos.data_ptr(), ctx.slot_mapping.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                      HM.ptr(v_first), v_first.stride(0) if v_first is not None else 0, HM.ptr(lam),
+                                      q.data_ptr(), T, _dev(qkv)))
+    return q
+
+
+USE_TILES = True       # bf16 attention on the matrix cores where the shape allows (tests compare both forms)
+
+
+def paged_attention(q, k_cache, v_cache, ctx: StepContext, scale, sink=None, window=0, keep_first=0, force_rows=False):
+    """q [T, H, D] over the paged caches k [blocks, block_size, G, D], v [blocks, block_size, G, V]; query head h reads
+    key/value head h // (H/G).  The token at position i sees key j <= i, and with window > 0 only if i - j < window or
+    j < keep_first.  ``sink`` f32 [H]: one more term exp(sink[h]) in the softmax denominator, without a value (zeros
+    = a sink of score 0).  Scores and weights are float32.  Returns [T, H * V]."""
+    if not q.is_cuda:
+        return cpu_ops.paged_attention(q, k_cache, v_cache, ctx, scale, sink, window, keep_first)
+    HM.require_cuda(q, k_cache.dtype, "q")
+    T, H, D = q.shape
+    bs, G, V = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    mb = ctx.block_tables.shape[1]
+    o = torch.empty((T, H * V), dtype=q.dtype, device=q.device)
+    lib = HM.load()
+    HM.check(lib.hm_attn_rows(HM.dtype_code(q.dtype), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                              ctx.block_tables.data_ptr(), ctx.tok_seq.data_ptr(), ctx.tok_pos.data_ptr(), HM.ptr(sink),
+                              int(window), int(keep_first), float(scale), o.data_ptr(), T, H, G, D, V, bs, mb, _dev(q)))
+    return o
+
+
+def delta_prepare(proj, cols, w2, w0, a_bias, H, D, decay_scale, unit_eps=1e-6):
+    """The float32 inputs of a delta-rule recurrence from the mixer's merged product.  cols = ((offset, size) of r, k, the
+    removal gate's pre-activation, and the decay's inner activation z) in proj's columns.  Per token, head and channel:
+      decay = exp(-decay_scale * sigmoid(w2 tanh(z) + w0)),  a = sigmoid(a_pre + a_bias),  u = k / sqrt(sum k^2 + unit_eps)
+    Returns f32 [T, H, 5, D] = decay, a * u, u, k, r."""
+    if not proj.is_cuda:
+        return cpu_ops.delta_prepare(proj, cols, w2, w0, a_bias, H, D, decay_scale)
+    _rows(proj, "proj")
+    T = proj.shape[0]
+    (r_off, _), (k_off, _), (a_off, _), (z_off, rank) = cols
+    assert w2.shape == (H * D, rank) and w2.is_contiguous() and w2.dtype == proj.dtype
+    prep = torch.empty((T, H, 5, D), dtype=torch.float32, device=proj.device)
+    HM.check(HM.load().hm_delta_prepare(HM.dtype_code(proj.dtype), proj.data_ptr(), proj.stride(0), r_off, k_off, a_off, z_off,
+                                        w2.data_ptr(), w0.data_ptr(), a_bias.data_ptr(), rank, float(decay_scale), float(unit_eps),
+                                        prep.data_ptr(), T, H, D, _dev(proj)))
+    return prep
+
+
+def delta_recurrence(prep, v, state, ctx: StepContext):
+    """Generalized delta rule over every sequence's portion, token after token, per head with a float32 state S [D, D]:
+      S <- diag(decay) S - (a u)(u^T S) + k v^T  (both terms read the old S),  o = S^T r.
+    state f32 [slots, H, D, D] is read at a portion's start (zero at position 0) and left at its end.  v [T, H*D] may be a
+    column slice.  Returns o f32 [T, H, D]."""
+    if not prep.is_cuda:
+        return cpu_ops.delta_recurrence(prep, v, state, ctx)
+    _rows(v, "v")
+    T, H, _, D = prep.shape
+    assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, D, D)
+    o = torch.empty((T, H, D), dtype=torch.float32, device=prep.device)
+    HM.check(HM.load().hm_delta_recurrence(HM.dtype_code(v.dtype), prep.data_ptr(), v.data_ptr(), v.stride(0), state.data_ptr(),
+                                           ctx.qstart.data_ptr(), ctx.seq_pos0.data_ptr(), ctx.seq_slot.data_ptr(), o.data_ptr(),
+                                           ctx.num_seqs, H, D, _dev(prep)))
+    return o
+
+
+def delta_gate_norm(o, g, norm_w, eps, dtype):
+    """o f32 [T, H, D] -> every head divided by its RMS, times norm_w [H*D], times sigmoid(g) (g [T, H*D], rows may be a
+    column slice), in ``dtype``."""
+    if not o.is_cuda:
+        return cpu_ops.delta_gate_norm(o, g, norm_w, eps, dtype)
+    _rows(g, "g")
+    T, H, D = o.shape
+    out = torch.empty((T, H * D), dtype=dtype, device=o.device)
+    HM.check(HM.load().hm_delta_gate_norm(HM.dtype_code(dtype), o.data_ptr(), g.data_ptr(), g.stride(0), norm_w.data_ptr(),
+                                          float(eps), out.data_ptr(), T, H, D, _dev(o)))
+    return out
+
+
+def relu_squared(z):
+    """max(z, 0)^2; z [T, F] may be a column slice of a wider product."""
+    if not z.is_cuda:
+        return cpu_ops.relu_squared(z)
+    _rows(z, "z")
+    T, Fw = z.shape
+    out = torch.empty((T, Fw), dtype=z.dtype, device=z.device)
+    HM.check(HM.load().hm_relu_squared(HM.dtype_code(z.dtype), z.data_ptr(), z.stride(0), out.data_ptr(), T, Fw, _dev(z)))
+    return out

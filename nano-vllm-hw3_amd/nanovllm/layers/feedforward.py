@@ -55,3 +55,19 @@ class RoutedExperts(nn.Module):
         idx, wts = seq_ops.moe_route(h, self.router, self.top, self.groups, self.keep)
         shared = self.shared(h) if self.shared is not None else None
         return seq_ops.moe_experts(h, idx, wts, self.w_gu, self.w_down, self.limit, self.alpha, shared, tiled=self._tiled)
+
+
+class ReluSquaredMLP(nn.Module):
+    """down(relu(up(h))^2).  ``extra_rows`` more rows of the up product belong to the caller (a gate that reads the same
+    h): forward returns (result, those columns of the product)."""
+
+    def __init__(self, width: int, ff: int, extra_rows: int = 0):
+        super().__init__()
+        self.ff = ff
+        self.up = nn.Parameter(torch.empty(ff + extra_rows, width), requires_grad=False)
+        self.down = nn.Parameter(torch.empty(width, ff), requires_grad=False)
+
+    def forward(self, h):
+        from nanovllm import hy_ops
+        z = F.linear(h, self.up)
+        return F.linear(hy_ops.relu_squared(z[:, :self.ff]), self.down), z[:, self.ff:]

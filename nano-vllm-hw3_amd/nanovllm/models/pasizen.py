@@ -66,6 +66,7 @@ class PasizenLayer(nn.Module):
 class PasizenForCausalLM(nn.Module):
     runs_portions = True           # stepped with portions; owns a latent cache and convolution state per layer run
     default_block_size = 64
+    native_library = "seqmix"
 
     @staticmethod
     def normalize_config(d: dict) -> dict:
@@ -209,6 +210,11 @@ class PasizenForCausalLM(nn.Module):
                                 device=device)
             for layer in self.layers:
                 layer.canon.state = state
+
+    def workspaces(self):
+        """Scratch buffers that captured decode graphs address."""
+        from nanovllm import _seqmix
+        return [_seqmix.decode_workspace]
 
     # ------------------------------------------------------------------ forward
     def forward(self, input_ids, positions, trace=None):

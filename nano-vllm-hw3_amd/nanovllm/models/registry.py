@@ -10,6 +10,7 @@ _MODELS = {
     "Qwen3ForCausalLM": ("nanovllm.models.qwen3", "Qwen3ForCausalLM"),
     "Qwen2ForCausalLM": ("nanovllm.models.qwen3", "Qwen3ForCausalLM"),      # the same decoder with qkv biases
     "Pasizen": ("nanovllm.models.pasizen", "PasizenForCausalLM"),
+    "Lipelix": ("nanovllm.models.lipelix", "LipelixForCausalLM"),
 }
 DEFAULT = "Qwen3ForCausalLM"
 
