@@ -84,6 +84,19 @@ int hm_attn_rows(int dtype, const void* q, const void* k_cache, const void* v_ca
                  const int32_t* tok_seq, const int32_t* tok_pos, const float* sink, int window, int keep_first, float scale,
                  void* o, int64_t T, int H, int G, int D, int V, int block_size, int max_blocks, void* stream);
 
+/* The same attention on the matrix cores, bf16 storage only, dim and vdim multiples of 8 up to 128, block_size % 64 == 0.
+ * Portions of any length (max_q = the longest portion of the step): */
+int hm_attn_tiles(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables, const int32_t* qstart,
+                  const int32_t* seq_pos0, const float* sink, int window, int keep_first, float scale, void* o, int B, int max_q,
+                  int H, int G, int D, int V, int block_size, int max_blocks, void* stream);
+/* Single-token queries (q [B, H, D], ctx[b] = keys of sequence b incl. the new one): the visible key tiles are split
+ * over `splits` workgroups per (sequence, key/value head) and merged in split order by a second launch.  At most 32
+ * query heads per key/value head.  workspace: hm_attn_decode_workspace_bytes(B, H, V, splits) bytes. */
+size_t hm_attn_decode_workspace_bytes(int64_t B, int H, int V, int splits);
+int hm_attn_decode(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables, const int32_t* ctx,
+                   const float* sink, int window, int keep_first, float scale, void* o, int64_t B, int H, int G, int D, int V,
+                   int block_size, int max_blocks, int splits, void* workspace, size_t workspace_bytes, void* stream);
+
 /* prep [T, H, 5, D] f32 = decay | a*u | u | k | r from the columns r_off, k_off, a_off (H*D wide) and z_off (rank wide) of
  * proj:  decay = exp(-decay_scale * sigmoid(w2 tanh(z) + w0)), a = sigmoid(a_pre + a_bias), u = k / sqrt(sum k^2 + unit_eps)
  * per head.  w2 [H*D, rank]. */

@@ -27,6 +27,11 @@ SIGNATURES = {
                               _i64, _vp, _vp, _i64, _vp]),
     "hm_attn_rows": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _f, _vp, _i64, _int, _int, _int, _int, _int,
                             _int, _vp]),
+    "hm_attn_tiles": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _f, _vp, _int, _int, _int, _int, _int, _int, _int, _int,
+                             _vp]),
+    "hm_attn_decode_workspace_bytes": (_sz, [_i64, _int, _int, _int]),
+    "hm_attn_decode": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _f, _vp, _i64, _int, _int, _int, _int, _int, _int, _int,
+                              _vp, _sz, _vp]),
     "hm_delta_prepare": (_int, [_int, _vp, _i64, _int, _int, _int, _int, _vp, _vp, _vp, _int, _f, _f, _vp, _i64, _int, _int, _vp]),
     "hm_delta_recurrence": (_int, [_int, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp]),
     "hm_delta_gate_norm": (_int, [_int, _vp, _vp, _i64, _vp, _f, _vp, _i64, _int, _int, _vp]),

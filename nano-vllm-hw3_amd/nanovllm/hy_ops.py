@@ -127,10 +127,31 @@ def paged_attention(q, k_cache, v_cache, ctx: StepContext, scale, sink=None, win
     mb = ctx.block_tables.shape[1]
     o = torch.empty((T, H * V), dtype=q.dtype, device=q.device)
     lib = HM.load()
+    tiles_ok = (USE_TILES and not force_rows and q.dtype == torch.bfloat16 and D % 8 == 0 and V % 8 == 0 and D <= 128 and
+                V <= 128 and bs % 64 == 0)
+    if tiles_ok and ctx.max_q == 1 and H // G <= 32:
+        splits = decode_splits(ctx.num_seqs * G, min(mb * bs, window + keep_first + 128) if window > 0 else mb * bs)
+        ws, n = HM.decode_workspace.get(q.device, lib.hm_attn_decode_workspace_bytes(T, H, V, splits))
+        HM.check(lib.hm_attn_decode(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), ctx.block_tables.data_ptr(),
+                                    ctx.ctx_lens.data_ptr(), HM.ptr(sink), int(window), int(keep_first), float(scale), o.data_ptr(),
+                                    T, H, G, D, V, bs, mb, splits, ws, n, _dev(q)))
+        return o
+    if tiles_ok:
+        HM.check(lib.hm_attn_tiles(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), ctx.block_tables.data_ptr(),
+                                   ctx.qstart.data_ptr(), ctx.seq_pos0.data_ptr(), HM.ptr(sink), int(window), int(keep_first),
+                                   float(scale), o.data_ptr(), ctx.num_seqs, ctx.max_q, H, G, D, V, bs, mb, _dev(q)))
+        return o
     HM.check(lib.hm_attn_rows(HM.dtype_code(q.dtype), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                               ctx.block_tables.data_ptr(), ctx.tok_seq.data_ptr(), ctx.tok_pos.data_ptr(), HM.ptr(sink),
                               int(window), int(keep_first), float(scale), o.data_ptr(), T, H, G, D, V, bs, mb, _dev(q)))
     return o
+
+
+def decode_splits(num_groups, max_keys):
+    """Splits of the key tiles in decode attention: about four workgroups per CU, at least two 64-key tiles per split.
+    Depends only on the batch size and the cache geometry, never on the sequences' lengths."""
+    want = max(1, 1024 // max(1, num_groups))
+    return int(max(1, min(want, (max_keys + 127) // 128, 64)))
 
 
 def delta_prepare(proj, cols, w2, w0, a_bias, H, D, decay_scale, unit_eps=1e-6):

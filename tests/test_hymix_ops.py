@@ -326,3 +326,29 @@ def test_delta_state_is_float32_over_long_runs(device, dtype):
         out.append(hy_ops.delta_recurrence(prep_in[a:e].contiguous().to(device), v[a:e].to(device), state, ctx))
         a, i = e, i + 1
     near(torch.cat(out), ref, torch.float32, f32=2e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,D,V", [(4, 4, 48, 48), (8, 2, 64, 128), (6, 1, 128, 8), (3, 3, 8, 40), (64, 2, 16, 16)])
+@pytest.mark.parametrize("window,keep", [(0, 0), (72, 20), (130, 0), (5, 200)])
+def test_matrix_core_attention_equals_portable_form(H, G, D, V, window, keep):
+    """bf16: the tile kernel (portions) and the split-key kernel (single tokens) against the portable kernel on the same
+    cache, for head sizes on and off the padded tile sizes, grouped heads, windows around tile borders; sequences whose
+    portions start inside a block, a batch of single tokens at unequal lengths."""
+    g = gen(H * D + window)
+    dev, bf, bs = "cuda", torch.bfloat16, 64
+    lens = [333, 64, 1, 129, 700]
+    need = [(n + bs - 1) // bs for n in lens]
+    perm = torch.randperm(sum(need) + 1, generator=g).tolist()
+    tables = [[perm.pop() for _ in range(k)] for k in need]
+    kc = rnd(g, sum(need) + 1, bs, G, D, dtype=bf).to(dev)
+    vc = rnd(g, sum(need) + 1, bs, G, V, dtype=bf).to(dev)
+    sink = rnd(g, H, s=2.0).to(dev)
+    for parts in ([(b, 0, n) for b, n in enumerate(lens)], [(0, 300, 333), (3, 127, 129), (4, 1, 700)],
+                  [(b, n - 1, n) for b, n in enumerate(lens)], [(4, 699, 700)]):
+        ctx = step_context(tables, parts, bs, dev)
+        q = rnd(g, ctx.num_tokens, H, D, dtype=bf).to(dev)
+        for sk in (sink, None):
+            ref = hy_ops.paged_attention(q, kc, vc, ctx, 0.3, sk, window, keep, force_rows=True)
+            got = hy_ops.paged_attention(q, kc, vc, ctx, 0.3, sk, window, keep)
+            near(got, ref.double().cpu(), bf, bf16=1.5e-2)
