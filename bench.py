@@ -399,8 +399,10 @@ def main():
     ap.add_argument("--model", default="0.6b", choices=sorted(MODELS),
                     help="0.6b = the headline benchmark; the larger models are experiments on the same workload")
     ap.add_argument("--families", nargs="*", metavar="SIZE", default=None,
-                    help="instead of the headline benchmark: prefill / decode throughput of the Pasizen family beside Qwen3 "
-                         "at equal layer sizes (w1024 w2048 w4096; default the first two) and the kernel-by-kernel roofline table")
+                    help="instead of the headline benchmark: prefill / decode throughput of another model family (--family) "
+                         "beside Qwen3 at equal layer sizes (w1024 w2048 w4096; default the first two) and the kernel-by-kernel "
+                         "roofline table")
+    ap.add_argument("--family", default="pasizen", choices=["pasizen", "lipelix"], help="the family --families measures")
     ap.add_argument("--backend", default="nccl", choices=["nccl", "gloo"],
                     help="gloo = rehearsal of the multi-rank path on fewer GPUs than ranks (ranks share devices)")
     args = ap.parse_args()
@@ -408,7 +410,7 @@ def main():
     if args.families is not None:
         from nanovllm.utils import family_bench
         torch.cuda.set_device(0)
-        print(json.dumps(family_bench.main(tuple(args.families) or ("w1024", "w2048"))), flush=True)
+        print(json.dumps(family_bench.main(tuple(args.families) or ("w1024", "w2048"), family=args.family)), flush=True)
         return
     rank = int(os.environ.get("RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))

@@ -2,6 +2,8 @@
 // (state slot, head).  Three launches: the float32 inputs of the recurrence from the mixer's merged product (parallel
 // over tokens), the recurrence (sequential over a portion's tokens, parallel over sequences, heads and value channels),
 // and the per-head norm and output gate (parallel over tokens).
+#include <algorithm>
+
 #include "hm_common.h"
 
 namespace hm {
@@ -26,7 +28,16 @@ __global__ void delta_prepare_kernel(const T* __restrict__ proj, int64_t row_str
         a = sigmoid_f(to_f(row[a_off + c]) + to_f(a_bias[c]));
         float acc = 0.f;
         const T* wr = w2 + (size_t)c * rank;
-        for (int j = 0; j < rank; ++j) acc += to_f(wr[j]) * tz[j];
+        struct alignas(sizeof(T) * 8) Pack { T v[8]; };
+        int j = 0;
+        if (rank % 8 == 0) {                   // 16-byte loads of the row (bf16); the order of the sum stays 0, 1, 2, ...
+            for (; j < rank; j += 8) {
+                const Pack pk = *(const Pack*)(wr + j);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc += to_f(pk.v[e]) * tz[j + e];
+            }
+        }
+        for (; j < rank; ++j) acc += to_f(wr[j]) * tz[j];
         decay = expf(-decay_scale * sigmoid_f(acc + to_f(w0[c])));
     }
     const float ss = block_sum(k * k, red);
@@ -41,75 +52,123 @@ __global__ void delta_prepare_kernel(const T* __restrict__ proj, int64_t row_str
     }
 }
 
-// One wave per (sequence, head, 64 value channels); a thread owns one column of S (DK >= D key channels in registers).
-// The five per-token vectors are staged in LDS (two buffers, one barrier per token) and read as broadcasts.
-template <typename T, int DK>
-__global__ __launch_bounds__(64) void delta_recurrence_kernel(const float* __restrict__ prep, const T* __restrict__ v,
-                                                              int64_t v_stride, float* __restrict__ state,
-                                                              const int32_t* __restrict__ qstart,
-                                                              const int32_t* __restrict__ seq_pos0,
-                                                              const int32_t* __restrict__ seq_slot, float* __restrict__ o,
-                                                              int H, int D) {
-    __shared__ float buf[2][5 * DK];
+// One workgroup of 256 threads per (sequence, head, 256 / SL value channels).  A column of S (one value channel, DK >= D
+// key channels) is spread over SL neighbouring lanes, DK / SL channels each in registers; u^T S and S^T r are summed over
+// those lanes with a butterfly, so every lane holds the total and the order of the sums is fixed by DK and SL alone.
+// The per-token vectors (decay, a u, u, k, r and v, DK floats each, zero beyond D) are staged in LDS CH tokens at a time:
+// the next chunk is requested from global memory before the current chunk's tokens run and written to the other buffer
+// after them, so the recurrence itself waits for LDS only, with one barrier per chunk.
+template <typename T, int DK, int SL, int CH>
+__global__ __launch_bounds__(256) void delta_recurrence_kernel(const float* __restrict__ prep, const T* __restrict__ v,
+                                                               int64_t v_stride, float* __restrict__ state,
+                                                               const int32_t* __restrict__ qstart,
+                                                               const int32_t* __restrict__ seq_pos0,
+                                                               const int32_t* __restrict__ seq_slot, float* __restrict__ o,
+                                                               int H, int D) {
+    constexpr int KS = DK / SL, COLS = 256 / SL, TOK = 6 * DK, NR = (CH * TOK + 255) / 256;
+    __shared__ __attribute__((aligned(16))) float buf[2][CH * TOK];
     const int b = blockIdx.x, hd = blockIdx.y;
     const int q0 = qstart[b], n = qstart[b + 1] - q0;
     if (n <= 0) return;
-    const int lane = threadIdx.x;
-    const int j = blockIdx.z * 64 + lane;
+    const int tid = threadIdx.x, slice = tid % SL, col = tid / SL;
+    const int j = blockIdx.z * COLS + col;
     const bool live = j < D;
     float* st = state + ((size_t)seq_slot[b] * H + hd) * (size_t)D * D;
-    float s[DK];
+    float s[KS];
     const bool fresh = seq_pos0[b] == 0;       // a sequence's first tokens: the state starts at zero, whatever the slot holds
 #pragma unroll
-    for (int i = 0; i < DK; ++i) s[i] = (!fresh && live && i < D) ? st[(size_t)i * D + j] : 0.f;
-
-    auto stage = [&](int tok, int which) {     // rows beyond D are zero: they leave their registers at zero
-        const float* src = prep + ((size_t)(q0 + tok) * H + hd) * 5 * D;
-        for (int e = lane; e < 5 * DK; e += 64) {
-            const int part = e / DK, i = e - part * DK;
-            buf[which][e] = i < D ? src[part * D + i] : 0.f;
+    for (int ii = 0; ii < KS; ++ii) {
+        const int i = slice * KS + ii;
+        s[ii] = (!fresh && live && i < D) ? st[(size_t)i * D + j] : 0.f;
+    }
+    float regs[NR];
+    auto request = [&](int tok0) {             // the vectors of tokens tok0 .. tok0 + CH - 1 into registers
+#pragma unroll
+        for (int k = 0; k < NR; ++k) {
+            const int e = tid + 256 * k;
+            const int tc = e / TOK, rem = e - tc * TOK, part = rem / DK, i = rem - part * DK, tok = tok0 + tc;
+            float val = 0.f;
+            if (e < CH * TOK && tok < n && i < D) {
+                const size_t row = (size_t)(q0 + tok);
+                val = part < 5 ? prep[(row * H + hd) * 5 * D + (size_t)part * D + i] : to_f(v[row * v_stride + hd * D + i]);
+            }
+            regs[k] = val;
         }
     };
-    stage(0, 0);
-    __syncthreads();
-    for (int tok = 0; tok < n; ++tok) {
-        const int cur = tok & 1;
-        if (tok + 1 < n) stage(tok + 1, cur ^ 1);
-        const float* p = buf[cur];
-        const float vj = live ? to_f(v[(size_t)(q0 + tok) * v_stride + hd * D + j]) : 0.f;
-        float dot = 0.f;
+    auto deposit = [&](int which) {
 #pragma unroll
-        for (int i = 0; i < DK; ++i) dot += p[2 * DK + i] * s[i];
-        float out = 0.f;
-#pragma unroll
-        for (int i = 0; i < DK; ++i) {
-            s[i] = p[i] * s[i] - p[DK + i] * dot + p[3 * DK + i] * vj;
-            out += s[i] * p[4 * DK + i];
+        for (int k = 0; k < NR; ++k) {
+            const int e = tid + 256 * k;
+            if (e < CH * TOK) buf[which][e] = regs[k];
         }
-        if (live) o[((size_t)(q0 + tok) * H + hd) * D + j] = out;
-        __syncthreads();
+    };
+    request(0);
+    deposit(0);
+    __syncthreads();
+    int which = 0;
+    for (int tok0 = 0; tok0 < n; tok0 += CH) {
+        const bool more = tok0 + CH < n;
+        if (more) request(tok0 + CH);
+        const int m = min(CH, n - tok0);
+        for (int tc = 0; tc < m; ++tc) {
+            const float* p = buf[which] + tc * TOK + slice * KS;
+            float dot = 0.f;
+#pragma unroll
+            for (int ii = 0; ii < KS; ++ii) dot += p[2 * DK + ii] * s[ii];
+#pragma unroll
+            for (int w = 1; w < SL; w <<= 1) dot += __shfl_xor(dot, w);
+            const float vj = buf[which][tc * TOK + 5 * DK + min(j, DK - 1)];
+            float out = 0.f;
+#pragma unroll
+            for (int ii = 0; ii < KS; ++ii) {
+                s[ii] = p[ii] * s[ii] - p[DK + ii] * dot + p[3 * DK + ii] * vj;
+                out += s[ii] * p[4 * DK + ii];
+            }
+#pragma unroll
+            for (int w = 1; w < SL; w <<= 1) out += __shfl_xor(out, w);
+            if (live && slice == 0) o[((size_t)(q0 + tok0 + tc) * H + hd) * D + j] = out;
+        }
+        if (more) {
+            deposit(which ^ 1);                // the other buffer was last read one chunk ago, before that chunk's barrier
+            __syncthreads();
+            which ^= 1;
+        }
     }
     if (live) {
 #pragma unroll
-        for (int i = 0; i < DK; ++i)
-            if (i < D) st[(size_t)i * D + j] = s[i];
+        for (int ii = 0; ii < KS; ++ii) {
+            const int i = slice * KS + ii;
+            if (i < D) st[(size_t)i * D + j] = s[ii];
+        }
     }
 }
 
-template <typename T>
-__global__ __launch_bounds__(64) void delta_gate_norm_kernel(const float* __restrict__ o, const T* __restrict__ g,
-                                                             int64_t g_stride, const T* __restrict__ norm_w, float eps,
-                                                             T* __restrict__ out, int H, int D) {
+// A head's D channels are spread over LPH lanes (a power of two, VEC consecutive channels per lane and round), so a wave
+// covers 64 / LPH heads of one token at once; a workgroup of four waves walks the token's heads.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void delta_gate_norm_kernel(const float* __restrict__ o, const T* __restrict__ g,
+                                                              int64_t g_stride, const T* __restrict__ norm_w, float eps,
+                                                              T* __restrict__ out, int H, int D, int LPH) {
     const int64_t t = blockIdx.x;
-    const int hd = blockIdx.y, lane = threadIdx.x;
-    const float* orow = o + ((size_t)t * H + hd) * D;
-    float ss = 0.f;
-    for (int i = lane; i < D; i += 64) ss += orow[i] * orow[i];
-    ss = wave_sum(ss);
-    const float r = 1.f / sqrtf(ss / (float)D + eps);
-    for (int i = lane; i < D; i += 64) {
-        const int c = hd * D + i;
-        out[(size_t)t * H * D + c] = from_f<T>(orow[i] * r * to_f(norm_w[c]) * sigmoid_f(to_f(g[(size_t)t * g_stride + c])));
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int per_wave = 64 / LPH, sub = lane / LPH, li = lane % LPH;
+    for (int hd = (blockIdx.y * 4 + wave) * per_wave + sub; hd < H + sub; hd += gridDim.y * 4 * per_wave) {
+        const bool head = hd < H;              // lanes of a head beyond the last still take part in the shuffles
+        const float* orow = o + ((size_t)t * H + (head ? hd : 0)) * D;
+        float ss = 0.f;
+        if (head)
+            for (int i = li * VEC; i < D; i += LPH * VEC)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) ss += orow[i + e] * orow[i + e];
+        for (int w = 1; w < LPH; w <<= 1) ss += __shfl_xor(ss, w);
+        if (!head) continue;
+        const float r = 1.f / sqrtf(ss / (float)D + eps);
+        for (int i = li * VEC; i < D; i += LPH * VEC)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const int c = hd * D + i + e;
+                out[(size_t)t * H * D + c] = from_f<T>(orow[i + e] * r * to_f(norm_w[c]) * sigmoid_f(to_f(g[(size_t)t * g_stride + c])));
+            }
     }
 }
 
@@ -140,14 +199,15 @@ extern "C" int hm_delta_prepare(int dtype, const void* proj, int64_t row_stride,
 template <typename DT>
 static int launch_recurrence(const float* prep, const void* v, int64_t v_stride, float* state, const int32_t* qstart,
                              const int32_t* seq_pos0, const int32_t* seq_slot, float* o, int B, int H, int D, hipStream_t s) {
-    dim3 grid((unsigned)B, (unsigned)H, (unsigned)((D + 63) / 64));
-#define HM_RECUR(DK)                                                                                                       \
-    hipLaunchKernelGGL((delta_recurrence_kernel<DT, DK>), grid, dim3(64), 0, s, prep, (const DT*)v, v_stride, state, qstart, \
-                       seq_pos0, seq_slot, o, H, D)
-    if (D <= 32) HM_RECUR(32);
-    else if (D <= 64) HM_RECUR(64);
-    else if (D <= 128) HM_RECUR(128);
-    else HM_RECUR(256);
+    constexpr int SL = 8, COLS = 256 / SL;
+    dim3 grid((unsigned)B, (unsigned)H, (unsigned)((D + COLS - 1) / COLS));
+#define HM_RECUR(DK, CH)                                                                                                      \
+    hipLaunchKernelGGL((delta_recurrence_kernel<DT, DK, SL, CH>), grid, dim3(256), 0, s, prep, (const DT*)v, v_stride, state, \
+                       qstart, seq_pos0, seq_slot, o, H, D)
+    if (D <= 32) HM_RECUR(32, 8);
+    else if (D <= 64) HM_RECUR(64, 8);
+    else if (D <= 128) HM_RECUR(128, 8);
+    else HM_RECUR(256, 4);
 #undef HM_RECUR
     return 0;
 }
@@ -173,12 +233,19 @@ extern "C" int hm_delta_gate_norm(int dtype, const float* o, const void* g, int6
         set_error("hm_delta_gate_norm: bad argument");
         return HM_EINVAL;
     }
-    if (H > 65535) { set_error("hm_delta_gate_norm: heads <= 65535"); return HM_ESHAPE; }
     if (T == 0) return HM_OK;
-    dim3 grid((unsigned)T, (unsigned)H);
+    const int vec = D % 4 == 0 ? 4 : 1;
+    int lph = 1;
+    while (lph < 64 && lph * vec < D) lph <<= 1;
+    const int heads_per_block = 4 * (64 / lph);
+    dim3 grid((unsigned)T, (unsigned)std::min(64, (H + heads_per_block - 1) / heads_per_block));
     HM_DISPATCH(dtype, "hm_delta_gate_norm",
-                hipLaunchKernelGGL(delta_gate_norm_kernel<DT>, grid, dim3(64), 0, as_stream(stream), o, (const DT*)g, g_stride,
-                                   (const DT*)norm_w, eps, (DT*)out, H, D));
+                if (vec == 4)
+                    hipLaunchKernelGGL((delta_gate_norm_kernel<DT, 4>), grid, dim3(256), 0, as_stream(stream), o, (const DT*)g,
+                                       g_stride, (const DT*)norm_w, eps, (DT*)out, H, D, lph);
+                else
+                    hipLaunchKernelGGL((delta_gate_norm_kernel<DT, 1>), grid, dim3(256), 0, as_stream(stream), o, (const DT*)g,
+                                       g_stride, (const DT*)norm_w, eps, (DT*)out, H, D, lph));
     HM_CHECK_LAUNCH("hm_delta_gate_norm");
     return HM_OK;
 }

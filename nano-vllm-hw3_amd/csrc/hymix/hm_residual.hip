@@ -1,6 +1,8 @@
 // The float32 residual of a decoder whose sublayers are normalised on both sides and gated: scaled embedding, the
 // boundary between two sublayers (gate, norm of the result, residual add, norm in front of the next sublayer, and the
 // row a token shift carries to the next step) in one launch per token, the token shift itself, and squared ReLU.
+#include <algorithm>
+
 #include "hm_common.h"
 
 namespace hm {
@@ -76,20 +78,29 @@ __global__ __launch_bounds__(256) void sublayer_close_kernel(float* __restrict__
     }
 }
 
-template <typename T>
+// VEC consecutive channels per thread (VEC = 8 when W % 8 == 0: 16-byte accesses for bf16)
+template <typename T, int VEC>
 __global__ void token_shift_kernel(const T* __restrict__ h, const T* __restrict__ mu, const T* __restrict__ state,
                                    int64_t slot_stride, const int32_t* __restrict__ tok_seq,
                                    const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ qstart,
                                    const int32_t* __restrict__ seq_slot, T* __restrict__ out, int W) {
+    struct alignas(sizeof(T) * VEC) Pack { T v[VEC]; };
     const int64_t t = blockIdx.x;
     const int b = tok_seq[t];
     const T* prev = nullptr;                   // position 0: nothing before it, whatever the slot holds
     if (tok_pos[t] > 0) prev = t > (int64_t)qstart[b] ? h + (size_t)(t - 1) * W : state + (size_t)seq_slot[b] * slot_stride;
     const T* hr = h + (size_t)t * W;
-    for (int c = threadIdx.x; c < W; c += blockDim.x) {
-        const float v = to_f(hr[c]);
-        const float p = prev ? to_f(prev[c]) : 0.f;
-        out[(size_t)t * W + c] = from_f<T>(v + (p - v) * to_f(mu[c]));
+    for (int c = threadIdx.x * VEC; c < W; c += blockDim.x * VEC) {
+        const Pack x = *(const Pack*)(hr + c), m = *(const Pack*)(mu + c);
+        Pack p, r;
+        if (prev) p = *(const Pack*)(prev + c);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const float v = to_f(x.v[e]);
+            const float pv = prev ? to_f(p.v[e]) : 0.f;
+            r.v[e] = from_f<T>(v + (pv - v) * to_f(m.v[e]));
+        }
+        *(Pack*)(out + (size_t)t * W + c) = r;
     }
 }
 
@@ -148,9 +159,16 @@ extern "C" int hm_token_shift(int dtype, const void* h, const void* mu, const vo
         return HM_EINVAL;
     }
     if (T == 0) return HM_OK;
+    // packs need aligned rows: the width and the slots' distance in whole packs
+    const bool wide = W % 8 == 0 && slot_stride % 8 == 0;
     HM_DISPATCH(dtype, "hm_token_shift",
-                hipLaunchKernelGGL(token_shift_kernel<DT>, dim3((unsigned)T), dim3(256), 0, as_stream(stream), (const DT*)h,
-                                   (const DT*)mu, (const DT*)state, slot_stride, tok_seq, tok_pos, qstart, seq_slot, (DT*)out, W));
+                if (wide)
+                    hipLaunchKernelGGL((token_shift_kernel<DT, 8>), dim3((unsigned)T), dim3(std::min(256, (W / 8 + 63) / 64 * 64)), 0,
+                                       as_stream(stream), (const DT*)h, (const DT*)mu, (const DT*)state, slot_stride, tok_seq,
+                                       tok_pos, qstart, seq_slot, (DT*)out, W);
+                else
+                    hipLaunchKernelGGL((token_shift_kernel<DT, 1>), dim3((unsigned)T), dim3(256), 0, as_stream(stream), (const DT*)h,
+                                       (const DT*)mu, (const DT*)state, slot_stride, tok_seq, tok_pos, qstart, seq_slot, (DT*)out, W));
     HM_CHECK_LAUNCH("hm_token_shift");
     return HM_OK;
 }

@@ -1,6 +1,6 @@
-"""Throughput of the Pasizen family beside the Qwen3 decoder at equal size (random weights, bf16, one GPU), and the
-time of every libseqmix kernel beside the like kernel of the Qwen3 path with both against their rooflines.
-Used by ``bench.py --families``; prints one JSON object."""
+"""Throughput of the Pasizen or the Lipelix family beside the Qwen3 decoder at equal size (random weights, bf16, one
+GPU), and the time of every libseqmix / libhymix kernel beside the like kernel of the Qwen3 path with both against their
+rooflines.  Used by ``bench.py --families [--family NAME]``; prints one JSON object."""
 import json
 import os
 import tempfile
@@ -37,6 +37,19 @@ def pasizen_config(width, heads, ff, layers, rank):
                         for i in range(layers)])
 
 
+def lipelix_config(width, heads, ff, layers):
+    """Full attention, windowed attention, delta rule, full attention, and so on; grouped heads as the Qwen3 model of the
+    size has them (heads / 2 key/value heads of 128), half of every head rotated, 512-token windows that keep 4 tokens,
+    delta-rule heads of 64 over the model's width."""
+    full = dict(heads=heads, kv_heads=max(1, heads // 2), dim=128, vdim=128, rot=dict(dims=64, base=10000.0), scale=128 ** -0.5,
+                v_mix=True)
+    kinds = [("attention", full), ("attention_2", dict(full, mask=dict(size=512, keep_first=4))),
+             ("general_delta", dict(heads=width // 64, dim=64, decay_rank=64)), ("attention", full)]
+    return dict(architecture="Lipelix", vocab=VOCAB, width=width, norm=dict(eps=1e-5), residual_mult=0.5, embedding=dict(scale=1.0),
+                max_positions=8192,
+                layers=[dict(type=kinds[i % 4][0], mixer=kinds[i % 4][1], mlp=dict(kind="dense", ff=ff)) for i in range(layers)])
+
+
 def _model_dir(cfg):
     d = tempfile.mkdtemp(prefix="family_bench_")
     with open(os.path.join(d, "config.json"), "w") as f:
@@ -60,7 +73,8 @@ def engine_throughput(family, size, prefill_seqs=8, prefill_len=1024, decode_seq
     from nanovllm import LLM
     from nanovllm.engine.sequence import ACTIVE, Sequence
     width, heads, ff, layers, rank = SIZES[size]
-    cfg = pasizen_config(width, heads, ff, layers, rank) if family == "pasizen" else qwen3_config(width, heads, ff, layers)
+    cfg = (pasizen_config(width, heads, ff, layers, rank) if family == "pasizen" else
+           lipelix_config(width, heads, ff, layers) if family == "lipelix" else qwen3_config(width, heads, ff, layers))
     llm = LLM(_model_dir(cfg), load_format="dummy", enforce_eager=False, max_model_len=2048,
               max_num_seqs=decode_seqs, max_num_batched_tokens=prefill_seqs * prefill_len, gpu_memory_utilization=0.5)
     g = torch.Generator().manual_seed(0)
@@ -74,7 +88,7 @@ def engine_throughput(family, size, prefill_seqs=8, prefill_len=1024, decode_seq
             out.append(s)
         return out
     res = {}
-    if family == "pasizen":
+    if family != "qwen3":
         pre = seqs_of(prefill_seqs, prefill_len)
         for s in pre:
             assert sch.reserve_portion(s, prefill_len)
@@ -243,11 +257,129 @@ def kernel_table(width=2048, heads=16, rank=256, ff=6144, T=8192, seq=1024, B=64
     return rows
 
 
-def main(sizes=("w1024", "w2048"), kernels=True):
+def hymix_kernel_table(width=2048, heads=16, ff=6144, T=8192, seq=1024, B=64, ctx=1024, window=512, keep=4):
+    """Seconds per launch of every libhymix kernel at a layer's size, its bound and the fraction of it reached; beside each
+    the like kernel of the Qwen3 path."""
+    from nanovllm import hy_ops, ops, seq_ops
+    dev, bf = "cuda", torch.bfloat16
+    rows = []
+
+    def add(name, like, sec, bytes_=0, flops=0):
+        bound = max(bytes_ / (HBM_GBPS * 1e9), flops / (MFMA_TFLOPS * 1e12))
+        rows.append(dict(kernel=name, like=like, us=round(sec * 1e6, 1), bound_us=round(bound * 1e6, 1),
+                         of_roofline=round(bound / sec, 3), bound="flops" if flops / (MFMA_TFLOPS * 1e12) > bytes_ / (HBM_GBPS * 1e9) else "bytes"))
+    r = lambda *s: torch.randn(*s, device=dev).to(bf)  # noqa: E731
+    nseq, bs, G, D = T // seq, 64, heads // 2, 128
+    import numpy as np
+
+    def context(portions):
+        tables, nxt = [], 0
+        for p0, n in portions:
+            nb = (p0 + n + bs - 1) // bs
+            tables.append(list(range(nxt, nxt + nb)))
+            nxt += nb
+        tok_seq = np.concatenate([np.full(n, b) for b, (_, n) in enumerate(portions)])
+        tok_pos = np.concatenate([np.arange(p0, p0 + n) for p0, n in portions])
+        slot = np.concatenate([np.asarray(tables[b])[np.arange(p0, p0 + n) // bs] * bs + np.arange(p0, p0 + n) % bs
+                               for b, (p0, n) in enumerate(portions)])
+        mb = max(len(t) for t in tables)
+        bt = np.zeros((len(portions), mb), dtype=np.int32)
+        for b, t in enumerate(tables):
+            bt[b, :len(t)] = t
+        qs = np.concatenate([[0], np.cumsum([n for _, n in portions])])
+        i32 = lambda v: torch.tensor(np.asarray(v), dtype=torch.int32, device=dev)  # noqa: E731
+        return seq_ops.StepContext(tok_seq=i32(tok_seq), tok_pos=i32(tok_pos), qstart=i32(qs), seq_pos0=i32([p for p, _ in portions]),
+                                   ctx_lens=i32([p + n for p, n in portions]), seq_slot=i32(list(range(len(portions)))),
+                                   slot_mapping=i32(slot), block_tables=i32(bt), num_seqs=len(portions), num_tokens=int(qs[-1]),
+                                   max_q=max(n for _, n in portions), block_size=bs, qstart_host=qs.tolist()), nxt
+    pre, nblk_p = context([(0, seq)] * nseq)
+    dec, nblk_d = context([(ctx - 1, 1)] * B)
+    nblk = max(nblk_p, nblk_d)
+    # ---- sublayer boundary | Qwen3: residual add + RMS norm
+    x, y, gate, gb, pw, nw = torch.randn(T, width, device=dev), r(T, width), r(T, width), r(width), r(width), r(width)
+    src, state = r(T, width), torch.zeros(nseq + 1, 1, width, device=dev, dtype=bf)
+    add("hm_sublayer_close (T=%d)" % T, "ql_add_rmsnorm",
+        _event_time(lambda: hy_ops.sublayer_close(x, y, gate, gb, pw, 0.5, nw, 1e-5, bf, carry=(src, state, 0, pre))),
+        bytes_=T * width * (8 + 2 + 2 + 2))
+    x2, res = r(T, width), r(T, width)
+    add("ql_add_rmsnorm (T=%d)" % T, "-", _event_time(lambda: ops.add_rmsnorm(x2, res, nw, 1e-6)), bytes_=T * width * 8)
+    # ---- elementwise launches | Qwen3: SiLU * mul
+    h, mu = r(T, width), r(width)
+    add("hm_token_shift (T=%d)" % T, "ql_silu_mul", _event_time(lambda: hy_ops.token_shift(h, mu, state, 0, pre)), bytes_=T * width * 4)
+    z = r(T, ff + width)
+    add("hm_relu_squared (T=%d, ff=%d)" % (T, ff), "ql_silu_mul", _event_time(lambda: hy_ops.relu_squared(z[:, :ff])), bytes_=T * ff * 4)
+    gu = r(T, 2 * ff)
+    add("ql_silu_mul (T=%d)" % T, "-", _event_time(lambda: ops.silu_mul(gu)), bytes_=T * ff * 6)
+    # ---- q/k/v preparation | Qwen3: per-head q/k norm + RoPE + K/V store
+    kc, vc = r(nblk, bs, G, D), r(nblk, bs, G, D)
+    qkv = r(T, (heads + 2 * G) * D)
+    qw, kw = r(heads * D), r(G * D)
+    inv_freq = hy_ops.rotary_inv_freq(64, 1e4, dev)
+    vf, lam = r(T, G * D), torch.tensor([0.3], device=dev)
+    add("hm_qkv_prepare (T=%d, proj norm, v mix)" % T, "ql_qknorm_rope_store",
+        _event_time(lambda: hy_ops.qkv_prepare(qkv, heads, G, D, D, qw, kw, 1e-5, inv_freq, False, pre, kc, vc, vf, lam)),
+        bytes_=T * ((heads + 2 * G) * D * 4 + G * D * 2))
+    add("hm_qkv_prepare (T=%d, unit norm)" % T, "ql_qknorm_rope_store",
+        _event_time(lambda: hy_ops.qkv_prepare(qkv, heads, G, D, D, None, None, 1e-5, inv_freq, True, pre, kc, vc, None, None)),
+        bytes_=T * (heads + 2 * G) * D * 4)
+    cos_sin = torch.randn(T, D, device=dev)
+    kq, vq = r(nblk * bs // 256 + 1, 256, G, D), r(nblk * bs // 256 + 1, 256, G, D)
+    add("ql_qknorm_rope_store (T=%d)" % T, "-",
+        _event_time(lambda: ops.qknorm_rope_store(qkv, None, cos_sin, qw[:D].contiguous(), kw[:D].contiguous(), 1e-6, heads, G, D, kq, vq,
+                                                  pre.slot_mapping, want_kv=False)), bytes_=T * (heads + 2 * G) * D * 4)
+    # ---- attention, prefill
+    q = r(T, heads, D)
+    sink = torch.randn(heads, device=dev)
+    pairs = nseq * seq * (seq + 1) / 2 * heads
+    add("hm_attn_tiles full (%dx%d, H=%d/%d, D=128)" % (nseq, seq, heads, G), "ql_attn_prefill",
+        _event_time(lambda: hy_ops.paged_attention(q, kc, vc, pre, 0.09, sink), 5), flops=pairs * 4 * D)
+    wpairs = nseq * heads * sum(min(i + 1, window) + min(keep, max(0, i + 1 - window)) for i in range(seq))
+    add("hm_attn_tiles window %d+%d (%dx%d)" % (window, keep, nseq, seq), "ql_attn_prefill",
+        _event_time(lambda: hy_ops.paged_attention(q, kc, vc, pre, 0.09, sink, window, keep), 5), flops=wpairs * 4 * D)
+    k, v = r(T, G, D), r(T, G, D)
+    cu = torch.arange(0, T + 1, seq, dtype=torch.int32, device=dev)
+    add("ql_attn_prefill (%dx%d, H=%d/%d, D=128)" % (nseq, seq, heads, G), "-", _event_time(lambda: ops.attn_prefill(q, k, v, cu, seq, 0.09), 5),
+        flops=pairs * 4 * D)
+    # ---- attention, decode
+    qd = r(B, heads, D)
+    add("hm_attn_decode full (B=%d, ctx=%d, G=%d)" % (B, ctx, G), "ql_paged_attn_decode",
+        _event_time(lambda: hy_ops.paged_attention(qd, kc, vc, dec, 0.09, sink)), bytes_=B * ctx * G * D * 4)
+    add("hm_attn_decode window %d+%d (B=%d, ctx=%d)" % (window, keep, B, ctx), "ql_paged_attn_decode",
+        _event_time(lambda: hy_ops.paged_attention(qd, kc, vc, dec, 0.09, sink, window, keep)), bytes_=B * (window + keep) * G * D * 4)
+    nb = (ctx + 255) // 256
+    kc2, vc2 = r(B * nb, 256, G, D), r(B * nb, 256, G, D)
+    tables = torch.arange(B * nb, dtype=torch.int32, device=dev).view(B, nb)
+    lens = torch.full((B,), ctx, dtype=torch.int32, device=dev)
+    ops.reserve_attn_workspace(B, heads, G, 256, nb, dev)
+    add("ql_paged_attn_decode (B=%d, ctx=%d, G=%d)" % (B, ctx, G), "-",
+        _event_time(lambda: ops.paged_attn_decode(qd, kc2, vc2, tables, lens, 0.09)), bytes_=B * ctx * G * D * 4)
+    # ---- delta rule: heads of 64 over the width
+    Hd, Dd, rank = width // 64, 64, 64
+    hd = Hd * Dd
+    proj = r(T, 5 * hd + rank)
+    w2, w0, ab, onw = r(hd, rank), r(hd), r(hd), r(hd)
+    cols = ((0, hd), (hd, hd), (4 * hd, hd), (5 * hd, rank))
+    add("hm_delta_prepare (T=%d, H=%d, D=%d)" % (T, Hd, Dd), "ql_qknorm_rope_store",
+        _event_time(lambda: hy_ops.delta_prepare(proj, cols, w2, w0, ab, Hd, Dd, 0.6)), bytes_=T * (hd * 6 + hd * 20))
+    prep = hy_ops.delta_prepare(proj, cols, w2, w0, ab, Hd, Dd, 0.6)
+    st = torch.zeros(max(nseq, B), Hd, Dd, Dd, device=dev)
+    vv = proj[:, 2 * hd:3 * hd]
+    add("hm_delta_recurrence prefill (%dx%d)" % (nseq, seq), "ql_attn_prefill", _event_time(lambda: hy_ops.delta_recurrence(prep, vv, st, pre), 5),
+        bytes_=T * hd * 26, flops=0)
+    prep_d = prep[:B].contiguous()
+    add("hm_delta_recurrence decode (B=%d)" % B, "ql_paged_attn_decode", _event_time(lambda: hy_ops.delta_recurrence(prep_d, vv[:B], st, dec)),
+        bytes_=B * Hd * Dd * Dd * 8)
+    o = torch.randn(T, Hd, Dd, device=dev)
+    add("hm_delta_gate_norm (T=%d)" % T, "ql_silu_mul", _event_time(lambda: hy_ops.delta_gate_norm(o, proj[:, 3 * hd:4 * hd], onw, 1e-5, bf)),
+        bytes_=T * hd * 8)
+    return rows
+
+
+def main(sizes=("w1024", "w2048"), kernels=True, family="pasizen"):
     out = dict(metric="family comparison", dtype="bf16", data="synthetic (random weights)", throughput=[], kernels=[])
     for size in sizes:
-        for family in ("pasizen", "qwen3"):
-            out["throughput"].append(engine_throughput(family, size))
+        for fam in (family, "qwen3"):
+            out["throughput"].append(engine_throughput(fam, size))
     if kernels:
-        out["kernels"] = kernel_table()
+        out["kernels"] = kernel_table() if family == "pasizen" else hymix_kernel_table()
     return out
