@@ -8,47 +8,73 @@
 
 namespace hm {
 
-// One workgroup per (token, head), one thread per key channel.  prep[t, h] = decay | a*u | u | k | r, D floats each.
+// One workgroup per (kPrepTokens consecutive tokens, head), one thread per key channel: a thread's row of w2 is read once
+// for the tokens of the tile.  prep[t, h] = decay | a*u | u | k | r, D floats each.
+constexpr int kPrepTokens = 8;
+
 template <typename T>
 __global__ void delta_prepare_kernel(const T* __restrict__ proj, int64_t row_stride, int r_off, int k_off, int a_off, int z_off,
                                      const T* __restrict__ w2, const T* __restrict__ w0, const T* __restrict__ a_bias, int rank,
-                                     float decay_scale, float unit_eps, float* __restrict__ prep, int H, int D) {
-    extern __shared__ float tz[];              // rank floats: tanh of the decay's inner projection
+                                     float decay_scale, float unit_eps, float* __restrict__ prep, int64_t T_, int H, int D) {
+    extern __shared__ float tz[];              // kPrepTokens x rank floats: tanh of the decay's inner projection
     __shared__ float red[16];
-    const int64_t t = blockIdx.x;
+    const int64_t t0 = (int64_t)blockIdx.x * kPrepTokens;
+    const int nt = (int)min((int64_t)kPrepTokens, T_ - t0);
     const int hd = blockIdx.y, i = threadIdx.x;
-    const T* row = proj + (size_t)t * row_stride;
-    for (int j = threadIdx.x; j < rank; j += blockDim.x) tz[j] = tanhf(to_f(row[z_off + j]));
+    for (int e = threadIdx.x; e < nt * rank; e += blockDim.x) {
+        const int tt = e / rank, j = e - tt * rank;
+        tz[e] = tanhf(to_f(proj[(size_t)(t0 + tt) * row_stride + z_off + j]));
+    }
     __syncthreads();
     const int c = hd * D + i;
-    float k = 0.f, r = 0.f, a = 0.f, decay = 0.f;
+    float acc[kPrepTokens];
+#pragma unroll
+    for (int tt = 0; tt < kPrepTokens; ++tt) acc[tt] = 0.f;
+    float bias_a = 0.f, bias_w = 0.f;
     if (i < D) {
-        k = to_f(row[k_off + c]);
-        r = to_f(row[r_off + c]);
-        a = sigmoid_f(to_f(row[a_off + c]) + to_f(a_bias[c]));
-        float acc = 0.f;
         const T* wr = w2 + (size_t)c * rank;
         struct alignas(sizeof(T) * 8) Pack { T v[8]; };
         int j = 0;
-        if (rank % 8 == 0) {                   // 16-byte loads of the row (bf16); the order of the sum stays 0, 1, 2, ...
+        if (rank % 8 == 0) {                   // 16-byte loads of the row (bf16); every token's sum runs over j = 0, 1, 2, ...
             for (; j < rank; j += 8) {
                 const Pack pk = *(const Pack*)(wr + j);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) acc += to_f(pk.v[e]) * tz[j + e];
+                for (int e = 0; e < 8; ++e) {
+                    const float w = to_f(pk.v[e]);
+#pragma unroll
+                    for (int tt = 0; tt < kPrepTokens; ++tt) acc[tt] += w * tz[(tt < nt ? tt : 0) * rank + j + e];
+                }
             }
         }
-        for (; j < rank; ++j) acc += to_f(wr[j]) * tz[j];
-        decay = expf(-decay_scale * sigmoid_f(acc + to_f(w0[c])));
+        for (; j < rank; ++j) {
+            const float w = to_f(wr[j]);
+#pragma unroll
+            for (int tt = 0; tt < kPrepTokens; ++tt) acc[tt] += w * tz[(tt < nt ? tt : 0) * rank + j];
+        }
+        bias_a = to_f(a_bias[c]);
+        bias_w = to_f(w0[c]);
     }
-    const float ss = block_sum(k * k, red);
-    if (i < D) {
-        const float u = k / sqrtf(ss + unit_eps);
-        float* out = prep + ((size_t)t * H + hd) * 5 * D + i;
-        out[0] = decay;
-        out[D] = a * u;
-        out[2 * D] = u;
-        out[3 * D] = k;
-        out[4 * D] = r;
+#pragma unroll
+    for (int tt = 0; tt < kPrepTokens; ++tt) {
+        if (tt >= nt) break;                   // (uniform over the workgroup)
+        const T* row = proj + (size_t)(t0 + tt) * row_stride;
+        float k = 0.f, r = 0.f, a = 0.f, decay = 0.f;
+        if (i < D) {
+            k = to_f(row[k_off + c]);
+            r = to_f(row[r_off + c]);
+            a = sigmoid_f(to_f(row[a_off + c]) + bias_a);
+            decay = expf(-decay_scale * sigmoid_f(acc[tt] + bias_w));
+        }
+        const float ss = block_sum(k * k, red);
+        if (i < D) {
+            const float u = k / sqrtf(ss + unit_eps);
+            float* out = prep + ((size_t)(t0 + tt) * H + hd) * 5 * D + i;
+            out[0] = decay;
+            out[D] = a * u;
+            out[2 * D] = u;
+            out[3 * D] = k;
+            out[4 * D] = r;
+        }
     }
 }
 
@@ -184,14 +210,14 @@ extern "C" int hm_delta_prepare(int dtype, const void* proj, int64_t row_stride,
         set_error("hm_delta_prepare: bad argument");
         return HM_EINVAL;
     }
-    if (D > 256 || rank > 8192 || H > 65535) { set_error("hm_delta_prepare: dim <= 256, rank <= 8192, heads <= 65535"); return HM_ESHAPE; }
+    if (D > 256 || rank > 1024 || H > 65535) { set_error("hm_delta_prepare: dim <= 256, rank <= 1024, heads <= 65535"); return HM_ESHAPE; }
     if (T == 0) return HM_OK;
-    dim3 grid((unsigned)T, (unsigned)H);
+    dim3 grid((unsigned)((T + kPrepTokens - 1) / kPrepTokens), (unsigned)H);
     const int threads = (D + 63) / 64 * 64;
     HM_DISPATCH(dtype, "hm_delta_prepare",
-                hipLaunchKernelGGL(delta_prepare_kernel<DT>, grid, dim3(threads), (size_t)rank * 4, as_stream(stream),
+                hipLaunchKernelGGL(delta_prepare_kernel<DT>, grid, dim3(threads), (size_t)rank * 4 * kPrepTokens, as_stream(stream),
                                    (const DT*)proj, row_stride, r_off, k_off, a_off, z_off, (const DT*)w2, (const DT*)w0,
-                                   (const DT*)a_bias, rank, decay_scale, unit_eps, prep, H, D));
+                                   (const DT*)a_bias, rank, decay_scale, unit_eps, prep, T, H, D));
     HM_CHECK_LAUNCH("hm_delta_prepare");
     return HM_OK;
 }
