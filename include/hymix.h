@@ -107,9 +107,10 @@ int hm_delta_prepare(int dtype, const void* proj, int64_t row_stride, int r_off,
 /* For every sequence b and head, over the tokens of its portion in order:
  *   S <- diag(decay) S - (a u)(u^T S) + k v^T (both terms from the old S);  o[t] = S^T r
  * state f32 [slots, H, D, D] is read at the start unless seq_pos0[b] == 0 (then S = 0) and written at the end.
- * v [T, H*D] in the storage type, rows v_stride apart.  o f32 [T, H, D].  D <= 256. */
+ * v [T, H*D] in the storage type, rows v_stride apart.  o f32 [T, H, D].  D <= 256.  max_q = the longest portion of the
+ * step (a hint for staging: results do not depend on it). */
 int hm_delta_recurrence(int dtype, const float* prep, const void* v, int64_t v_stride, float* state, const int32_t* qstart,
-                        const int32_t* seq_pos0, const int32_t* seq_slot, float* o, int B, int H, int D, void* stream);
+                        const int32_t* seq_pos0, const int32_t* seq_slot, float* o, int B, int H, int D, int max_q, void* stream);
 
 /* out[t, h*D + i] = o[t, h, i] / sqrt(mean_i o[t, h]^2 + eps) * norm_w[h*D + i] * sigmoid(g[t, h*D + i]). */
 int hm_delta_gate_norm(int dtype, const float* o, const void* g, int64_t g_stride, const void* norm_w, float eps, void* out,

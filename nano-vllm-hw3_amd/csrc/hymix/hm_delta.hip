@@ -78,6 +78,15 @@ __global__ void delta_prepare_kernel(const T* __restrict__ proj, int64_t row_str
     }
 }
 
+// Sum over 8 neighbouring lanes with data-parallel-primitive moves (no LDS round trip): pairs, quads, then the mirrored
+// half row; every lane of the group ends with the same total.
+__device__ __forceinline__ float sum8(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+    return v;
+}
+
 // One workgroup of 256 threads per (sequence, head, 256 / SL value channels).  A column of S (one value channel, DK >= D
 // key channels) is spread over SL neighbouring lanes, DK / SL channels each in registers; u^T S and S^T r are summed over
 // those lanes with a butterfly, so every lane holds the total and the order of the sums is fixed by DK and SL alone.
@@ -91,6 +100,7 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(const float* __re
                                                                const int32_t* __restrict__ seq_pos0,
                                                                const int32_t* __restrict__ seq_slot, float* __restrict__ o,
                                                                int H, int D) {
+    static_assert(SL == 8, "the lane sums are written for groups of 8");
     constexpr int KS = DK / SL, COLS = 256 / SL, TOK = 6 * DK, NR = (CH * TOK + 255) / 256;
     __shared__ __attribute__((aligned(16))) float buf[2][CH * TOK];
     const int b = blockIdx.x, hd = blockIdx.y;
@@ -113,7 +123,9 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(const float* __re
         for (int k = 0; k < NR; ++k) {
             const int e = tid + 256 * k;
             const int tc = e / TOK, rem = e - tc * TOK, part = rem / DK, i = rem - part * DK, tok = tok0 + tc;
-            float val = 0.f;
+            // beyond the portion's end a chunk is filled with the identity step (decay 1, everything else 0): every chunk
+            // then runs CH steps of straight-line code and the state passes through the padding unchanged
+            float val = part == 0 && tok >= n ? 1.f : 0.f;
             if (e < CH * TOK && tok < n && i < D) {
                 const size_t row = (size_t)(q0 + tok);
                 val = part < 5 ? prep[(row * H + hd) * 5 * D + (size_t)part * D + i] : to_f(v[row * v_stride + hd * D + i]);
@@ -135,14 +147,13 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(const float* __re
     for (int tok0 = 0; tok0 < n; tok0 += CH) {
         const bool more = tok0 + CH < n;
         if (more) request(tok0 + CH);
-        const int m = min(CH, n - tok0);
-        for (int tc = 0; tc < m; ++tc) {
+#pragma unroll
+        for (int tc = 0; tc < CH; ++tc) {
             const float* p = buf[which] + tc * TOK + slice * KS;
             float dot = 0.f;
 #pragma unroll
             for (int ii = 0; ii < KS; ++ii) dot += p[2 * DK + ii] * s[ii];
-#pragma unroll
-            for (int w = 1; w < SL; w <<= 1) dot += __shfl_xor(dot, w);
+            dot = sum8(dot);
             const float vj = buf[which][tc * TOK + 5 * DK + min(j, DK - 1)];
             float out = 0.f;
 #pragma unroll
@@ -150,9 +161,8 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(const float* __re
                 s[ii] = p[ii] * s[ii] - p[DK + ii] * dot + p[3 * DK + ii] * vj;
                 out += s[ii] * p[4 * DK + ii];
             }
-#pragma unroll
-            for (int w = 1; w < SL; w <<= 1) out += __shfl_xor(out, w);
-            if (live && slice == 0) o[((size_t)(q0 + tok0 + tc) * H + hd) * D + j] = out;
+            out = sum8(out);
+            if (live && slice == 0 && tok0 + tc < n) o[((size_t)(q0 + tok0 + tc) * H + hd) * D + j] = out;
         }
         if (more) {
             deposit(which ^ 1);                // the other buffer was last read one chunk ago, before that chunk's barrier
@@ -224,13 +234,20 @@ extern "C" int hm_delta_prepare(int dtype, const void* proj, int64_t row_stride,
 
 template <typename DT>
 static int launch_recurrence(const float* prep, const void* v, int64_t v_stride, float* state, const int32_t* qstart,
-                             const int32_t* seq_pos0, const int32_t* seq_slot, float* o, int B, int H, int D, hipStream_t s) {
+                             const int32_t* seq_pos0, const int32_t* seq_slot, float* o, int B, int H, int D, int max_q,
+                             hipStream_t s) {
     constexpr int SL = 8, COLS = 256 / SL;
     dim3 grid((unsigned)B, (unsigned)H, (unsigned)((D + COLS - 1) / COLS));
 #define HM_RECUR(DK, CH)                                                                                                      \
     hipLaunchKernelGGL((delta_recurrence_kernel<DT, DK, SL, CH>), grid, dim3(256), 0, s, prep, (const DT*)v, v_stride, state, \
                        qstart, seq_pos0, seq_slot, o, H, D)
-    if (D <= 32) HM_RECUR(32, 8);
+    // single tokens (decode): one token staged at a time, so that many small workgroups fit a CU; the sums are the same
+    if (max_q <= 1) {
+        if (D <= 32) HM_RECUR(32, 1);
+        else if (D <= 64) HM_RECUR(64, 1);
+        else if (D <= 128) HM_RECUR(128, 1);
+        else HM_RECUR(256, 1);
+    } else if (D <= 32) HM_RECUR(32, 8);
     else if (D <= 64) HM_RECUR(64, 8);
     else if (D <= 128) HM_RECUR(128, 8);
     else HM_RECUR(256, 4);
@@ -240,7 +257,7 @@ static int launch_recurrence(const float* prep, const void* v, int64_t v_stride,
 
 extern "C" int hm_delta_recurrence(int dtype, const float* prep, const void* v, int64_t v_stride, float* state,
                                    const int32_t* qstart, const int32_t* seq_pos0, const int32_t* seq_slot, float* o, int B,
-                                   int H, int D, void* stream) {
+                                   int H, int D, int max_q, void* stream) {
     if (B < 0 || H < 1 || D < 1 || v_stride < (int64_t)H * D || (B > 0 && (!prep || !v || !state || !qstart || !seq_pos0 || !seq_slot || !o))) {
         set_error("hm_delta_recurrence: bad argument");
         return HM_EINVAL;
@@ -248,7 +265,7 @@ extern "C" int hm_delta_recurrence(int dtype, const float* prep, const void* v, 
     if (D > 256 || H > 65535) { set_error("hm_delta_recurrence: dim <= 256 and heads <= 65535"); return HM_ESHAPE; }
     if (B == 0) return HM_OK;
     HM_DISPATCH(dtype, "hm_delta_recurrence",
-                launch_recurrence<DT>(prep, v, v_stride, state, qstart, seq_pos0, seq_slot, o, B, H, D, as_stream(stream)));
+                launch_recurrence<DT>(prep, v, v_stride, state, qstart, seq_pos0, seq_slot, o, B, H, D, max_q, as_stream(stream)));
     HM_CHECK_LAUNCH("hm_delta_recurrence");
     return HM_OK;
 }

@@ -33,7 +33,7 @@ SIGNATURES = {
     "hm_attn_decode": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _f, _vp, _i64, _int, _int, _int, _int, _int, _int, _int,
                               _vp, _sz, _vp]),
     "hm_delta_prepare": (_int, [_int, _vp, _i64, _int, _int, _int, _int, _vp, _vp, _vp, _int, _f, _f, _vp, _i64, _int, _int, _vp]),
-    "hm_delta_recurrence": (_int, [_int, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp]),
+    "hm_delta_recurrence": (_int, [_int, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp]),
     "hm_delta_gate_norm": (_int, [_int, _vp, _vp, _i64, _vp, _f, _vp, _i64, _int, _int, _vp]),
     "hm_relu_squared": (_int, [_int, _vp, _i64, _vp, _i64, _int, _vp]),
 }

@@ -185,7 +185,7 @@ def delta_recurrence(prep, v, state, ctx: StepContext):
     o = torch.empty((T, H, D), dtype=torch.float32, device=prep.device)
     HM.check(HM.load().hm_delta_recurrence(HM.dtype_code(v.dtype), prep.data_ptr(), v.data_ptr(), v.stride(0), state.data_ptr(),
                                            ctx.qstart.data_ptr(), ctx.seq_pos0.data_ptr(), ctx.seq_slot.data_ptr(), o.data_ptr(),
-                                           ctx.num_seqs, H, D, _dev(prep)))
+                                           ctx.num_seqs, H, D, max(int(ctx.max_q), 1), _dev(prep)))
     return o
 
 

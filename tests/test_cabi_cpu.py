@@ -131,3 +131,44 @@ def test_seqmix_argument_validation_needs_no_gpu():
     assert lib.sm_latent_attn_decode(one, one, one, one, one, 0.1, 2, 4, 64, 64, 4, 2, one, 16, None) == -3   # workspace
     assert lib.sm_moe_route(1, one, one, one, one, 4, 64, 8, 3, 4, 1, None) == -2                        # top > keep * E/groups
     assert lib.sm_moe_grouped(one, one, one, one, one, None, 1.0, 1.7, one, 4, 2, 8, 60, 64, one, one, one, one, one, None) == -2
+
+
+# ---- libhymix (include/hymix.h) ----------------------------------------------------------------------------------------
+HYMIX_HEADER = os.path.join(ROOT, "include", "hymix.h")
+
+
+def hymix_declared():
+    src = re.sub(r"/\*.*?\*/", "", open(HYMIX_HEADER).read(), flags=re.S)
+    return sorted(set(re.findall(r"\b(hm_[a-z0-9_]+)\s*\(", src)))
+
+
+def test_hymix_binding_covers_header_and_library_exports_it():
+    from nanovllm import _hymix as HM
+    HM.build_if_missing()
+    lib = ctypes.CDLL(HM.LIB_PATH)
+    names = hymix_declared()
+    assert sorted(HM.SIGNATURES) == names
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in hymix.h but not exported"
+    assert HM.load().hm_version() >= 1
+
+
+def test_hymix_argument_validation_needs_no_gpu():
+    from nanovllm import _hymix as HM
+    lib = HM.load()
+    one = ctypes.c_void_p(16)   # never dereferenced: the calls below are rejected first
+    assert lib.hm_embed_scaled(7, one, one, 1.0, one, 4, 64, None) == -1                                  # unknown dtype
+    assert lib.hm_sublayer_close(1, one, one, None, 64, one, one, 0.5, None, 1e-5, None, None, None, 0, None, None, None, 4,
+                                 64, None) == -1                                                          # a result without its gate
+    assert lib.hm_sublayer_close(1, one, None, None, 0, None, None, 0.5, one, 1e-5, one, None, None, 0, None, None, None, 4,
+                                 1 << 20, None) == -2                                                     # wider than the row buffer
+    assert lib.hm_qkv_prepare(1, one, 100, 4, 3, 16, 8, None, None, 1e-5, one, 4, 0, one, one, one, one, None, 0, None, one, 4,
+                              None) == -1                                                                 # heads % kv_heads
+    assert lib.hm_qkv_prepare(1, one, 200, 4, 2, 16, 8, None, None, 1e-5, one, 9, 0, one, one, one, one, None, 0, None, one, 4,
+                              None) == -1                                                                 # rotation wider than a head
+    assert lib.hm_attn_tiles(one, one, one, one, one, one, None, 0, 0, 0.1, one, 2, 8, 4, 2, 20, 16, 64, 4, None) == -2   # dim % 8
+    assert lib.hm_attn_tiles(one, one, one, one, one, one, None, 0, 0, 0.1, one, 2, 8, 4, 2, 16, 16, 48, 4, None) == -2   # block % 64
+    assert lib.hm_attn_decode(one, one, one, one, one, None, 0, 0, 0.1, one, 2, 4, 2, 64, 64, 64, 4, 2, one, 16, None) == -3  # workspace
+    assert b"workspace" in lib.hm_last_error()
+    assert lib.hm_delta_recurrence(1, one, one, 10, one, one, one, one, one, 2, 2, 8, 1, None) == -1     # v rows narrower than heads * dim
+    assert lib.hm_delta_recurrence(1, one, one, 1024, one, one, one, one, one, 2, 2, 512, 1, None) == -2  # dim > 256
