@@ -5,8 +5,9 @@
 
 namespace hm {
 
-// One workgroup per token.  q and k travel through LDS as f32: [H*D] then [G*D].
-template <typename T>
+// One workgroup per token.  q and k travel through LDS as f32: [H*D] then [G*D].  VEC consecutive channels per global
+// access (VEC = 8 when every segment of the row starts and ends on a multiple of 8: 16-byte accesses for bf16).
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void qkv_prepare_kernel(const T* __restrict__ qkv, int64_t row_stride, int H, int G, int D,
                                                           int V, const T* __restrict__ q_norm_w, const T* __restrict__ k_norm_w,
                                                           float eps, const float* __restrict__ inv_freq, int rot_half,
@@ -20,12 +21,19 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(const T* __restrict__ 
     const int64_t t = blockIdx.x;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int nq = H * D, nk = G * D, nv = G * V;
+    struct alignas(sizeof(T) * VEC) Pack { T v[VEC]; };
     const T* row = qkv + (size_t)t * row_stride;
     float sq = 0.f, sk = 0.f;
-    for (int c = tid; c < nq + nk; c += 256) {
-        const float v = to_f(row[c]);
-        qk[c] = v;
-        if (c < nq) sq += v * v; else sk += v * v;
+    for (int c = tid * VEC; c < nq + nk; c += 256 * VEC) {
+        const Pack pk = *(const Pack*)(row + c);
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const float v = to_f(pk.v[e]);
+            qk[c + e] = v;
+            ss += v * v;
+        }
+        if (c < nq) sq += ss; else sk += ss;
     }
     if (q_norm_w != nullptr) {                 // RMS norm over the whole projection, with a weight
         sq = block_sum(sq, red);
@@ -34,12 +42,14 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(const T* __restrict__ 
         for (int c = tid; c < nq + nk; c += 256)
             qk[c] = c < nq ? qk[c] * rq * to_f(q_norm_w[c]) : qk[c] * rk * to_f(k_norm_w[c - nq]);
     }
-    __syncthreads();
+    // the angles depend on the channel pair alone: one sine and cosine per pair, shared by all heads
+    float* cs = qk + nq + nk;
     const float pos = (float)tok_pos[t];
+    for (int i = tid; i < rot_half; i += 256) sincosf(pos * inv_freq[i], cs + rot_half + i, cs + i);
+    __syncthreads();
     for (int e = tid; e < (H + G) * rot_half; e += 256) {       // one thread per rotated pair
         const int hh = e / rot_half, i = e - hh * rot_half;
-        float s, c;
-        sincosf(pos * inv_freq[i], &s, &c);
+        const float c = cs[i], s = cs[rot_half + i];
         float* p = qk + (size_t)hh * D;
         const float a = p[i], b = p[i + rot_half];
         p[i] = a * c - b * s;
@@ -57,18 +67,33 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(const T* __restrict__ 
         }
         __syncthreads();
     }
-    for (int c = tid; c < nq; c += 256) q_out[(size_t)t * nq + c] = from_f<T>(qk[c]);
+    for (int c = tid * VEC; c < nq; c += 256 * VEC) {
+        Pack pk;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) pk.v[e] = from_f<T>(qk[c + e]);
+        *(Pack*)(q_out + (size_t)t * nq + c) = pk;
+    }
     const int slot = slot_mapping[t];
     if (slot < 0) return;
-    for (int c = tid; c < nk; c += 256) k_cache[(size_t)slot * nk + c] = from_f<T>(qk[nq + c]);
+    for (int c = tid * VEC; c < nk; c += 256 * VEC) {
+        Pack pk;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) pk.v[e] = from_f<T>(qk[nq + c + e]);
+        *(Pack*)(k_cache + (size_t)slot * nk + c) = pk;
+    }
     const T* vr = row + nq + nk;
     if (v_first != nullptr) {
         const float l = lam[0];
         const T* fr = v_first + (size_t)t * v_first_stride;
-        for (int c = tid; c < nv; c += 256)
-            v_cache[(size_t)slot * nv + c] = from_f<T>((1.f - l) * to_f(vr[c]) + l * to_f(fr[c]));
+        for (int c = tid * VEC; c < nv; c += 256 * VEC) {
+            const Pack a = *(const Pack*)(vr + c), f = *(const Pack*)(fr + c);
+            Pack pk;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) pk.v[e] = from_f<T>((1.f - l) * to_f(a.v[e]) + l * to_f(f.v[e]));
+            *(Pack*)(v_cache + (size_t)slot * nv + c) = pk;
+        }
     } else {
-        for (int c = tid; c < nv; c += 256) v_cache[(size_t)slot * nv + c] = vr[c];
+        for (int c = tid * VEC; c < nv; c += 256 * VEC) *(Pack*)(v_cache + (size_t)slot * nv + c) = *(const Pack*)(vr + c);
     }
 }
 
@@ -168,14 +193,19 @@ extern "C" int hm_qkv_prepare(int dtype, const void* qkv, int64_t row_stride, in
         set_error("hm_qkv_prepare: bad argument");
         return HM_EINVAL;
     }
-    const size_t lds = (size_t)(H + G) * D * 4;
+    const size_t lds = ((size_t)(H + G) * D + 2 * (size_t)rot_half) * 4;
     if (lds > 60 * 1024) { set_error("hm_qkv_prepare: (heads + kv_heads) * dim = %d does not fit the row buffer", (H + G) * D); return HM_ESHAPE; }
     if (T == 0) return HM_OK;
-    HM_DISPATCH(dtype, "hm_qkv_prepare",
-                hipLaunchKernelGGL(qkv_prepare_kernel<DT>, dim3((unsigned)T), dim3(256), lds, as_stream(stream), (const DT*)qkv,
-                                   row_stride, H, G, D, V, (const DT*)q_norm_w, (const DT*)k_norm_w, eps, inv_freq, rot_half,
-                                   unit_norm, tok_pos, slot_mapping, (DT*)k_cache, (DT*)v_cache, (const DT*)v_first,
-                                   v_first_stride, lam, (DT*)q_out));
+    // packs need every segment (q, k, v, the rows themselves and the blended values' rows) on multiples of 8 elements
+    const bool wide = (H * D) % 8 == 0 && (G * D) % 8 == 0 && (G * V) % 8 == 0 && row_stride % 8 == 0 &&
+                      (!v_first || v_first_stride % 8 == 0);
+    const uintptr_t bits = (uintptr_t)qkv | (uintptr_t)v_first | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)v_cache;
+#define HM_PREP(VEC_)                                                                                                         \
+    hipLaunchKernelGGL((qkv_prepare_kernel<DT, VEC_>), dim3((unsigned)T), dim3(256), lds, as_stream(stream), (const DT*)qkv,  \
+                       row_stride, H, G, D, V, (const DT*)q_norm_w, (const DT*)k_norm_w, eps, inv_freq, rot_half, unit_norm,  \
+                       tok_pos, slot_mapping, (DT*)k_cache, (DT*)v_cache, (const DT*)v_first, v_first_stride, lam, (DT*)q_out)
+    HM_DISPATCH(dtype, "hm_qkv_prepare", if (wide && bits % (8 * sizeof(DT)) == 0) HM_PREP(8); else HM_PREP(1));
+#undef HM_PREP
     HM_CHECK_LAUNCH("hm_qkv_prepare");
     return HM_OK;
 }
