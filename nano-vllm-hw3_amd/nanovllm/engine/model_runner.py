@@ -1,6 +1,9 @@
 """Runs the model for one scheduler step on one GPU.  With tensor parallelism every rank is its own
 process (launched by torch.distributed.run) executing the SAME control flow on the same inputs; the
 only cross-rank traffic is the RCCL collectives inside the layers, so no RPC channel is needed."""
+import contextlib
+import gc
+
 import torch
 import torch.distributed as dist
 
@@ -10,6 +13,21 @@ from nanovllm.models import registry
 from nanovllm.models.qwen3 import AttnContext, set_context
 from nanovllm.utils.loader import init_dummy_weights, load_model
 from nanovllm.utils.quantization import apply_quant_from_config, reserve_workspace
+
+
+@contextlib.contextmanager
+def no_finalizers():
+    """No cyclic garbage collection inside: while a stream captures, the capturing thread may not free device memory or
+    destroy graphs and events, and that is what the finalizers of an engine that has just become garbage do.  A
+    collection that happens to start in the middle of a capture fails inside a destructor and aborts the process."""
+    gc.collect()
+    was_enabled = gc.isenabled()
+    gc.disable()
+    try:
+        yield
+    finally:
+        if was_enabled:
+            gc.enable()
 
 
 class ModelRunner:
@@ -152,7 +170,7 @@ class ModelRunner:
                 logits.copy_(self.model.compute_logits(self.model(ids, v[2])))
             seq_ops.set_step(step)
             try:
-                with torch.no_grad():
+                with torch.no_grad(), no_finalizers():
                     body()                                       # warm-up: sizes every workspace, settles lazy choices
                     torch.cuda.synchronize()
                     g = torch.cuda.CUDAGraph()
@@ -549,7 +567,7 @@ class ModelRunner:
             # tensor-parallel ranks: RCCL's watchdog thread polls events while this thread captures; a capture in
             # "thread_local" mode is not invalidated by what other threads of the process do
             mode = "thread_local" if self.world_size > 1 else "global"
-            with torch.cuda.graph(g, pool, capture_error_mode=mode):
+            with no_finalizers(), torch.cuda.graph(g, pool, capture_error_mode=mode):
                 step(bs)
             if pool is None:
                 pool = g.pool()
