@@ -81,7 +81,7 @@ class LipelixForCausalLM(nn.Module):
             # the rank of the decay's inner projection is a tensor's shape, not a config value: a default until the
             # checkpoint is seen (load_checkpoint_tensor resizes), or what a dummy model asks for
             if spec["type"] == "general_delta":
-                spec["decay_rank"] = spec["mixer"].get("decay_rank", 16)
+                spec["decay_rank"] = spec["mixer"].get("decay_rank", 32)
             layers.append(spec)
         d["layers"] = layers
         mixed = [(s["mixer"]["kv_heads"], s["mixer"]["vdim"]) for s in layers if s["type"] in ATTENTION_KINDS and s["mixer"].get("v_mix")]
